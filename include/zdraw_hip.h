@@ -1,0 +1,214 @@
+/*
+ * zdraw_hip.h: C ABI of the MI355X (gfx950) attention backend.
+ *
+ * This is the drop-in boundary for zdraw's DiT joint self-attention. It
+ * replaces the attention slice of the reference's Metal bridge
+ * (src/metal/metal_c.zig, implemented by src/metal/metal_api.m): opaque
+ * pointer handles, plain-old-data parameter structs passed by const pointer,
+ * int return codes. Each declaration cites the reference declaration it
+ * replaces (paths relative to the reference tree).
+ *
+ * Return-code convention (metal_api.m:3072-3079, 1103-1113, 6604-6607):
+ *    0  success
+ *   -1  no usable handle / launch could not be issued
+ *   -2  the device reported an error when the work completed
+ *    1  "unavailable": the shape or operands are outside what this backend
+ *       computes; NOTHING was enqueued and the caller takes its own fallback
+ *       (zdraw's attention_fast.run falls through to its CPU kernel on
+ *       error.UnsupportedShape, runtime/attention_fast.zig:16-23). The
+ *       fallback counter is bumped.
+ *    2  the operands are malformed for the declared shape (buffer too small,
+ *       misaligned offset, zero dimension): the caller's error.InvalidShape.
+ *
+ * Threading: one host thread per queue, as in the reference (counters are
+ * plain integers, metal_api.m:333). Work on one queue executes in order.
+ */
+#ifndef ZDRAW_HIP_H
+#define ZDRAW_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ZDRAW_HIP_OK 0
+#define ZDRAW_HIP_ERR_HANDLE (-1)
+#define ZDRAW_HIP_ERR_DEVICE (-2)
+#define ZDRAW_HIP_UNAVAILABLE 1
+#define ZDRAW_HIP_INVALID 2
+
+/* metal_c.zig:245-256 (AttnParams), 24 bytes, same field order. */
+typedef struct ZdrawAttnParams {
+    uint32_t tokens;
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t head_dim;
+    uint32_t causal;
+    uint32_t valid; /* keys >= valid are masked for every query; 0 = none */
+} ZdrawAttnParams;
+
+/* mattn.Kernel order (metal/mattn.zig:19, metal_api.m:2983). Only BLOCK is
+ * implemented by this backend: the bf16-MFMA flash kernel for head_dim 128. */
+enum { ZDRAW_HIP_K_ROWS = 0, ZDRAW_HIP_K_FLASH = 1, ZDRAW_HIP_K_BLOCK = 2, ZDRAW_HIP_K_WIDE = 3 };
+
+/* Element types of activations. */
+enum { ZDRAW_HIP_F32 = 0, ZDRAW_HIP_F16 = 1, ZDRAW_HIP_BF16 = 2 };
+
+/* What is applied to Q and K rows as they are loaded. */
+enum {
+    ZDRAW_HIP_QK_NONE = 0,  /* operands used as given (standalone attention) */
+    ZDRAW_HIP_QK_KLEIN = 1, /* krms_rope: klein/zflux2_glue_shader.zig:61-83 */
+    ZDRAW_HIP_QK_ZIMAGE = 2 /* qk_norm_rope: metal/mqk_shader.zig:46-97 */
+};
+
+/* Where K's norm+rope happens for the fused entry. */
+enum {
+    ZDRAW_HIP_K_IN_TILE_LOAD = 0, /* inside the attention kernel, per K tile */
+    ZDRAW_HIP_K_PREPASS = 1       /* one pre-pass kernel into library scratch, then attention */
+};
+
+/*
+ * Extension block for the fused entry (no counterpart struct in the
+ * reference: it gathers what RopeHmParams (klein/zflux2_glue_shader.zig:87-93),
+ * QkNormParams (metal_c.zig:258-274) and the in_off/out_off arguments of
+ * zdraw_metal_run_attention_steel_route_enc (metal_c.zig:339-349) carry).
+ * Strides are in ELEMENTS: [0]=between batch segments, [1]=between tokens,
+ * [2]=between heads; head_dim is contiguous.
+ */
+typedef struct ZdrawHipAttnExt {
+    uint64_t q_off, k_off, v_off, out_off; /* byte offsets into the buffers */
+    uint64_t q_stride[3];
+    uint64_t k_stride[3];
+    uint64_t v_stride[3];
+    uint64_t out_stride[3];
+    uint64_t rope_batch_rows;  /* rope-table / position rows between segments; 0 = shared */
+    uint64_t mask_batch_bytes; /* key_pad bytes between segments; 0 = shared */
+    uint64_t zimage_base[3];   /* Z-Image axis bases in pairs (zrope.Cache.axisBases) */
+    uint32_t zimage_dims[3];   /* Z-Image axis widths, sum = head_dim */
+    uint32_t batch;            /* independent segments, >= 1 */
+    uint32_t in_dtype;         /* ZDRAW_HIP_F32 or ZDRAW_HIP_BF16 */
+    uint32_t out_dtype;        /* ZDRAW_HIP_F32 or ZDRAW_HIP_BF16 */
+    uint32_t qk_mode;          /* ZDRAW_HIP_QK_* */
+    uint32_t k_site;           /* ZDRAW_HIP_K_IN_TILE_LOAD or ZDRAW_HIP_K_PREPASS */
+    uint32_t txt_rows;         /* tokens < txt_rows use the *_txt weights (Klein double block) */
+    float eps;                 /* RMSNorm epsilon */
+} ZdrawHipAttnExt;
+
+/* Buffer handles for the fused entry's side operands (NULL where unused). */
+typedef struct ZdrawHipQkOperands {
+    void* q_weight;     /* f32[128]  (norm_q) */
+    void* k_weight;     /* f32[128]  (norm_k) */
+    void* q_weight_txt; /* f32[128]  (norm_added_q) or NULL */
+    void* k_weight_txt; /* f32[128]  (norm_added_k) or NULL */
+    void* rope_cos;     /* Klein: f32 [rows][128] */
+    void* rope_sin;     /* Klein: f32 [rows][128] */
+    void* pos;          /* Z-Image: u64 [rows][3] (zrope.Pos) */
+    void* rope_pairs;   /* Z-Image: f32 (cos,sin) pairs (zrope.Cache.pairBytes) */
+    void* key_pad;      /* u8 [segments][tokens], nonzero = key excluded; NULL = no mask */
+} ZdrawHipQkOperands;
+
+/* ---- device / queue lifecycle ------------------------------------------ */
+/* metal_c.zig:8-11. NULL when no gfx950 device is usable
+ * (the caller's error.MetalNotAvailable). */
+void* zdraw_hip_create_device(void);
+void zdraw_hip_release_device(void* device);
+void* zdraw_hip_create_queue(void* device); /* one HIP stream, default priority */
+void zdraw_hip_release_queue(void* queue);
+
+/* ---- buffers (metal_c.zig:12-33) ----------------------------------------- */
+void* zdraw_hip_create_buffer(void* device, size_t size);
+void* zdraw_hip_create_buffer_with_data(void* device, const uint8_t* data, size_t size);
+/* Borrowed DEVICE memory (e.g. a tensor another runtime owns): never freed by
+ * release_buffer. The Metal call wraps host memory; on a discrete GPU the
+ * no-copy form only makes sense for memory already on the device. */
+void* zdraw_hip_create_buffer_no_copy(void* device, void* device_ptr, size_t size);
+void zdraw_hip_read_buffer(void* buffer, uint8_t* dst, size_t size);
+void zdraw_hip_write_buffer(void* buffer, const uint8_t* src, size_t size);
+size_t zdraw_hip_buffer_length(void* buffer);
+void* zdraw_hip_buffer_device_ptr(void* buffer); /* no reference counterpart: interop */
+void zdraw_hip_release_buffer(void* buffer);
+
+/* ---- pipelines (metal_c.zig:99-107) -------------------------------------- */
+/* The kernels are compiled ahead of time for gfx950, so "compile" is a lookup
+ * by entry name: "attention_block_mfma" (the only attention pipeline) and
+ * "qk_norm_rope". Unknown names return NULL and write a message. */
+void* zdraw_hip_compile(void* device, const char* entry, char* error_buf, size_t error_len);
+void zdraw_hip_release_pipeline(void* pipeline);
+size_t zdraw_hip_pipeline_threads(void* pipeline);
+
+/* ---- standalone attention (metal_c.zig:137-147) -------------------------- */
+/* q, k, v, output: f32 token-major [tokens][heads][head_dim] buffers, as the
+ * reference's. Blocks until the result is in `output`. */
+int zdraw_hip_run_attention(void* queue, void* pipeline, void* q, void* k, void* v, void* output,
+                            const ZdrawAttnParams* params, uint32_t kernel, size_t thread_count);
+
+/* ---- resident batch (metal_c.zig:286-311, 350) --------------------------- */
+void* zdraw_hip_batch_begin(void* queue);
+int zdraw_hip_run_attention_enc(void* batch, void* pipeline, void* q, void* k, void* v, void* o,
+                                const ZdrawAttnParams* params, uint32_t kernel, size_t thread_count);
+int zdraw_hip_run_attention_enc_off(void* batch, void* pipeline, void* q, void* k, void* v, void* o,
+                                    const ZdrawAttnParams* params, uint32_t kernel, size_t thread_count,
+                                    uint64_t in_off, uint64_t out_off);
+/* Waits for everything enqueued since batch_begin and frees the batch. */
+int zdraw_hip_batch_end(void* batch);
+
+/* ---- fused QK-norm + rope + attention ------------------------------------ */
+/* Replaces the rmsRopeHm x2..4 + zdraw_metal_run_attention_steel_route_enc
+ * sequence (klein/zflux2_resident.zig:1547-1550, 1673-1710; metal_c.zig:339-349)
+ * and mqk.run + attention for Z-Image (metal/mres.zig:47-80): Q and K arrive
+ * un-normalised, V as is; one launch (or pre-pass + launch) writes O. */
+int zdraw_hip_run_attention_fused_enc(void* batch, void* q, void* k, void* v, void* out,
+                                      const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                                      const ZdrawHipQkOperands* ops);
+/* Same, on a queue, blocking until complete. */
+int zdraw_hip_run_attention_fused(void* queue, void* q, void* k, void* v, void* out,
+                                  const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                                  const ZdrawHipQkOperands* ops);
+
+/* ---- standalone QK-norm + rope (metal_c.zig:148-159, QkNormParams :258-274) -
+ * In place on f32 token-major q [tokens][heads][128] and k [tokens][kv_heads][128].
+ * Only ext->qk_mode, eps, txt_rows, zimage_* and rope_batch_rows are read. */
+int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
+                               const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                               const ZdrawHipQkOperands* ops);
+
+/* ---- library-owned scratch (metal_c.zig:321-325) -------------------------- */
+/* Grow-only, process-lifetime, filled at (re)allocation with 0x00 (0xFF when
+ * ZDRAW_SCRATCH_POISON is set, metal_api.m:6147-6181). slot in [0, 5). */
+void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes);
+
+/* ---- counters and timing (metal_api.m:333-353, 420-433) ------------------- */
+void zdraw_hip_metrics_reset(void);
+uint64_t zdraw_hip_dispatch_count(void);
+uint64_t zdraw_hip_command_count(void);
+uint64_t zdraw_hip_attn_fallback_count(void);
+uint64_t zdraw_hip_gpu_ns(void); /* device time summed over completed batches / blocking runs */
+
+/* HIP events on a queue's stream, for measuring kernels where they run. */
+void* zdraw_hip_event_create(void);
+int zdraw_hip_event_record(void* event, void* queue);
+int zdraw_hip_event_sync(void* event);
+float zdraw_hip_event_elapsed_ms(void* start, void* stop); /* negative on error */
+void zdraw_hip_event_release(void* event);
+int zdraw_hip_queue_sync(void* queue);
+
+/* Tuning knob for measurements: waves per workgroup (4 or 8; 0 = default). */
+void zdraw_hip_set_attention_waves(int nwaves);
+
+/* ABI drift guard (src/abi_gen.zig, runtime/abi_assert.zig:29): sizeof of the
+ * shared structs as this library was compiled. which: 0 = ZdrawAttnParams,
+ * 1 = ZdrawHipAttnExt, 2 = ZdrawHipQkOperands. */
+size_t zdraw_hip_abi_sizeof(int which);
+/* Last error text of this thread's most recent failing call ("" if none). */
+const char* zdraw_hip_last_error(void);
+
+#define ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE 24
+#define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 208
+#define ZDRAW_HIP_ABI_QK_OPERANDS_SIZE 72
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,154 @@
+"""CPU-only checks of the boundary: the C-ABI library loads and exports every
+declared symbol, struct sizes match the header, and the host layer's error
+behaviour without a device follows the reference's contract. No GPU compute."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import zoracle as zo
+from zdraw_amd import hip, host, workloads as wl
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "zdraw_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(zdraw_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = hip.lib()
+    declared = header_symbols()
+    assert len(declared) >= 35
+    for name in declared:
+        assert hasattr(L, name), f"libzdraw_hip.so lacks {name}"
+    # the Python binding table and the header agree
+    assert sorted(hip.SYMBOLS) == declared
+
+
+def test_abi_struct_sizes():
+    L = hip.lib()
+    # AttnParams must stay 24 bytes (runtime/abi_assert.zig:29)
+    assert L.zdraw_hip_abi_sizeof(0) == 24 == C.sizeof(hip.AttnParams)
+    assert L.zdraw_hip_abi_sizeof(1) == C.sizeof(hip.AttnExt) == 208
+    assert L.zdraw_hip_abi_sizeof(2) == C.sizeof(hip.QkOperands) == 72
+    text = open(os.path.join(ROOT, "include", "zdraw_hip.h")).read()
+    assert "#define ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE 24" in text
+    assert "#define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 208" in text
+    assert "#define ZDRAW_HIP_ABI_QK_OPERANDS_SIZE 72" in text
+
+
+def test_pipeline_lookup_without_device_is_null():
+    L = hip.lib()
+    err = C.create_string_buffer(128)
+    assert not L.zdraw_hip_compile(None, b"attention_block_mfma", err, 128)
+
+
+def _has_gpu():
+    return os.path.exists("/dev/kfd")
+
+
+@pytest.mark.skipif(_has_gpu(), reason="device present")
+def test_context_init_reports_not_available_without_device():
+    # mattn_test.zig:9-12: error.MetalNotAvailable is how "no device" surfaces
+    with pytest.raises(host.NotAvailable):
+        host.Context.init()
+
+
+def _oracle_cpu(out, q, k, v, scratch, cfg):
+    try:
+        res = zo.attention_run(q, k, v, zo.Config(cfg.tokens, cfg.heads, cfg.kv_heads, cfg.head_dim,
+                                                  cfg.causal, cfg.valid), scratch_len=scratch.size)
+    except zo.OracleError:
+        return 1
+    out[:] = res.ravel()
+    return 0
+
+
+def test_attention_fast_without_backend_uses_callers_cpu_kernel():
+    # runtime/attention_fast.zig:15-23: metal == null -> attention.run
+    rng = np.random.default_rng(0)
+    cfg = host.Config(5, 2, 1, 8, causal=True)
+    q = rng.standard_normal((5, 2, 8), dtype=np.float32)
+    k = rng.standard_normal((5, 1, 8), dtype=np.float32)
+    v = rng.standard_normal((5, 1, 8), dtype=np.float32)
+    got = host.attention_fast_run(None, q, k, v, cfg, cpu=_oracle_cpu)
+    want = zo.attention_run(q, k, v, zo.Config(5, 2, 1, 8, True))
+    assert np.array_equal(got, want)
+
+
+def test_attention_fast_without_backend_and_without_cpu_fails_loudly():
+    cfg = host.Config(4, 1, 1, 128)
+    z = np.zeros((4, 1, 128), np.float32)
+    with pytest.raises(host.NotAvailable):
+        host.attention_fast_run(None, z, z, z, cfg, cpu=None)
+
+
+def test_attention_fast_propagates_cpu_shape_error():
+    cfg = host.Config(4, 1, 1, 8)
+    z = np.zeros((4, 1, 8), np.float32)
+    with pytest.raises(host.InvalidShape):
+        host.attention_fast_run(None, z, z, z, cfg, cpu=_oracle_cpu, scratch_len=1)
+
+
+def test_host_rope_tables_match_oracle_bitwise():
+    c, s = host.klein_build_rope_ref(5, 7, 2, 3, theta=2000.0, txt_len=16)
+    c2, s2 = zo.klein_build_rope_ref(5, 7, 2, 3, theta=2000.0, txt_len=16)
+    assert np.array_equal(c, c2) and np.array_equal(s, s2)
+    c, s = host.klein_build_rope_ref(64, 64, theta=10000.0)
+    c2, s2 = zo.klein_build_rope_ref(64, 64, theta=10000.0)
+    assert c.shape == (4608, 128) and np.array_equal(c, c2) and np.array_equal(s, s2)
+    vals, bases = host.zimage_rope_fill(wl.ZIMAGE_DIMS, wl.ZIMAGE_LENS, wl.ZIMAGE_THETA)
+    cfg = zo.RopeConfig(wl.ZIMAGE_DIMS, wl.ZIMAGE_LENS, wl.ZIMAGE_THETA)
+    assert np.array_equal(vals, zo.zrope_fill(cfg)) and bases == zo.zrope_axis_bases(cfg)
+    with pytest.raises(host.InvalidShape):
+        host.zimage_rope_fill((2, 3, 2), (1, 1, 1), 10.0)
+    with pytest.raises(host.InvalidShape):
+        host.zimage_rope_fill((2, 2, 2), (1, 1, 1), 0.0)
+
+
+def test_host_positions_follow_reference_sequence_order():
+    pos = host.zimage_sequence_positions(64, 64, 512)
+    assert pos.shape == (4608, 3)
+    assert np.array_equal(pos[:4096], zo.zseq_grid((1, 64, 64), (513, 0, 0)))
+    assert np.array_equal(pos[4096:], zo.zseq_grid((512, 1, 1), (1, 0, 0)))
+    # padding: 7x9 image -> 64 slots, 33 caption tokens -> 64 slots
+    pos = host.zimage_sequence_positions(7, 9, 33)
+    assert pos.shape == (128, 3)
+    assert pos[62].tolist() == [65, 6, 8] and pos[63].tolist() == [0, 0, 0]
+    assert pos[64].tolist() == [1, 0, 0] and pos[127].tolist() == [64, 0, 0]
+
+
+def test_bf16_rounding_helper_is_round_to_nearest_even():
+    x = np.array([1.0, 1.00390625, 1.01171875, -3.0e-39, 3.3e38], np.float32)
+    bits = host.f32_to_bf16_bits(x)
+    back = host.bf16_bits_to_f32(bits)
+    assert back[0] == 1.0
+    assert back[1] == 1.0            # 1 + 2^-8 is a tie -> even mantissa (1.0)
+    assert back[2] == 1.015625       # 1 + 3*2^-8 is a tie -> even mantissa (1 + 2^-6)
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(0)
+    y = rng.standard_normal(10000).astype(np.float32) * 100
+    want = torch.from_numpy(y).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(host.bf16_bits_to_f32(host.f32_to_bf16_bits(y)), want)
+
+
+def test_workload_flops_match_the_published_work_figures():
+    # 4 * S^2 * D * H (cmd/gemmbench.zig:5887): 260.92 GFLOP at Klein 1024^2
+    def flops(tokens, heads, batch=1, keys=None):
+        keys = [tokens] * batch if keys is None else keys
+        return 4.0 * 128 * heads * sum(tokens * k for k in keys)
+    assert abs(flops(4608, 24) / 1e9 - 260.92) < 0.01
+    assert abs(flops(1536, 24, 4) / 1e9 - 115.96) < 0.01
+    assert abs(flops(4608, 30) / 1e9 - 326.15) < 0.01
+    assert abs(flops(8704, 24, 2, [8704 - 435, 8704 - 212]) / 1e9 - 1792.67) < 0.01
+    w = wl.by_name("klein_edit_ragged", small=True)
+    assert w.key_pad.shape == (2, w.tokens) and w.key_pad[0, 13:200].all() and not w.key_pad[0, :13].any()
+    assert w.flops == 4.0 * 128 * w.heads * w.tokens * ((w.tokens - 187) + (w.tokens - 50))
+    w1 = wl.by_name("klein_1024", seed=3, small=True)
+    w2 = wl.by_name("klein_1024", seed=3, small=True)
+    assert np.array_equal(w1.q, w2.q) and np.array_equal(w1.v, w2.v)

@@ -1,0 +1,379 @@
+"""GPU parity tests: the HIP path (through the C ABI and the host layer above
+it) against the CPU oracle on the same seeded inputs.
+
+Tolerance of the bf16 path against the fp32 reference: max abs <= 2e-2 and
+mean abs <= 2e-3 (tests/refimpl.py). Run-to-run results must be bit-identical.
+"""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+from oracle import zoracle as zo
+from tests import refimpl
+from zdraw_amd import hip, host, workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = host.Context.init()
+    yield c
+    c.deinit()
+
+
+def oracle_cfg(cfg: host.Config) -> zo.Config:
+    return zo.Config(cfg.tokens, cfg.heads, cfg.kv_heads, cfg.head_dim, cfg.causal, cfg.valid)
+
+
+def oracle_cpu(out, q, k, v, scratch, cfg):
+    try:
+        res = zo.attention_run(q, k, v, oracle_cfg(cfg), scratch_len=scratch.size)
+    except zo.OracleError:
+        return 1
+    out[:] = res.ravel()
+    return 0
+
+
+# ------------------------------------------------ the reference's own test cases
+def test_context_init_and_pick(ctx):
+    # metal/mattn.zig:134-150: head_dim 128 gets the MFMA block kernel
+    p = ctx.pick(4608, 128)
+    assert p is not None and p["kernel"] == hip.K_BLOCK and p["threads"] in (256, 512)
+    assert ctx.pick(16, 256) is None and ctx.pick(16, 64) is None
+
+
+def test_tiny_reference_case_takes_the_fallback_contract(ctx):
+    # metal/mattn_test.zig:8-32 uses head_dim 2: outside the MFMA kernel, so the
+    # context refuses it and attention_fast.run lands on the caller's CPU kernel.
+    cfg = host.Config(2, 1, 1, 2)
+    q = [1.0, 0.0, 0.0, 1.0]
+    v = [2.0, 4.0, 6.0, 8.0]
+    before = hip.lib().zdraw_hip_dispatch_count()
+    with pytest.raises(host.UnsupportedShape):
+        ctx.run(q, q, v, cfg)
+    assert hip.lib().zdraw_hip_dispatch_count() == before  # nothing was enqueued
+    got = host.attention_fast_run(ctx, q, q, v, cfg, cpu=oracle_cpu)
+    want = zo.attention_run(q, q, v, oracle_cfg(cfg))
+    assert np.allclose(got, want, atol=1e-4)
+    with pytest.raises(host.UnsupportedShape):
+        host.attention_fast_run(ctx, q, q, v, cfg, cpu=None)
+
+
+# metal/mattn_test.zig:47-53 (block_cases): D=128, tails inside and across tiles
+BLOCK_CASES = [(16, 1), (48, 2), (53, 3), (288, 4), (289, 2)]
+
+
+@pytest.mark.parametrize("tokens,heads", BLOCK_CASES)
+def test_block_cases_match_cpu(ctx, tokens, heads):
+    say(f"block case tokens={tokens} heads={heads}")
+    rng = np.random.default_rng(tokens * 31 + heads)  # seed rule of mattn_test.zig:66
+    shape = (tokens, heads, 128)
+    q = rng.standard_normal(shape, dtype=np.float32) * 0.5
+    k = rng.standard_normal(shape, dtype=np.float32) * 0.5
+    v = rng.standard_normal(shape, dtype=np.float32) * 0.5
+    cfg = host.Config(tokens, heads, heads, 128)
+    want = zo.attention_run(q, k, v, oracle_cfg(cfg))
+    got = ctx.run(q, k, v, cfg)
+    mx, mean = refimpl.check_close(got, want, f"block {tokens}x{heads}")
+    say(f"  max abs {mx:.2e} mean abs {mean:.2e}")
+    # the reference accepts 2e-3 for its half-precision MMA kernel on these inputs
+    assert mx <= 4e-3
+    again = ctx.run(q, k, v, cfg)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    pooled = ctx.run_pooled(q, k, v, cfg)
+    assert np.array_equal(got.view(np.uint32), pooled.view(np.uint32))
+
+
+@pytest.mark.parametrize("tokens,heads,dim,kv,causal", [
+    (1, 2, 8, 2, False), (31, 2, 16, 1, False), (97, 3, 64, 3, True), (16, 1, 256, 1, False),
+    (40, 4, 128, 2, False), (40, 2, 128, 2, True),
+])
+def test_out_of_scope_shapes_are_refused_not_miscomputed(ctx, tokens, heads, dim, kv, causal):
+    # metal/mattn_test.zig:35-43 (flash_cases): GQA, causal, narrow and wide heads
+    rng = np.random.default_rng(1)
+    q = rng.standard_normal((tokens, heads, dim), dtype=np.float32)
+    k = rng.standard_normal((tokens, kv, dim), dtype=np.float32)
+    v = rng.standard_normal((tokens, kv, dim), dtype=np.float32)
+    cfg = host.Config(tokens, heads, kv, dim, causal)
+    with pytest.raises(host.UnsupportedShape):
+        ctx.run(q, k, v, cfg)
+    got = host.attention_fast_run(ctx, q, k, v, cfg, cpu=oracle_cpu)
+    assert np.array_equal(got, zo.attention_run(q, k, v, oracle_cfg(cfg)))
+
+
+def test_shape_errors(ctx):
+    z = np.zeros(2 * 2 * 128, np.float32)
+    with pytest.raises(host.UnsupportedShape):
+        ctx.run(z[:0], z[:0], z[:0], host.Config(0, 2, 2, 128))        # mattn.zig:383
+    with pytest.raises(host.InvalidShape):
+        ctx.run(z, z, z, host.Config(2, 0, 2, 128))
+    with pytest.raises(host.InvalidShape):
+        ctx.run(z, z[:-128], z, host.Config(2, 2, 2, 128))
+    with pytest.raises(host.InvalidShape):
+        ctx.run(z, z, z, host.Config(2, 2, 2, 128), out_len=z.size + 1)
+    with pytest.raises(host.InvalidShape):
+        ctx.run(z, z[:256], z[:256], host.Config(2, 3, 2, 128))       # heads % kv_heads
+
+
+@pytest.mark.parametrize("tokens,valid", [(3, 2), (100, 64), (100, 65), (130, 1), (257, 200)])
+def test_valid_limit_masks_trailing_keys(ctx, tokens, valid):
+    # runtime/attention.zig:135-156 semantics at head_dim 128
+    say(f"valid case tokens={tokens} valid={valid}")
+    rng = np.random.default_rng(tokens + valid)
+    shape = (tokens, 2, 128)
+    q, k, v = (rng.standard_normal(shape, dtype=np.float32) for _ in range(3))
+    k[valid:] *= 30.0  # a dropped mask would let these keys dominate
+    cfg = host.Config(tokens, 2, 2, 128, valid=valid)
+    got = ctx.run(q, k, v, cfg)
+    want = zo.attention_run(q, k, v, oracle_cfg(cfg))
+    refimpl.check_close(got, want, f"valid {tokens}/{valid}")
+
+
+# ---------------------------------------------------------- config 1: plumbing
+def test_config1_plumbing_through_attention_fast(ctx):
+    w = wl.by_name("plumbing")
+    cfg = host.Config(w.tokens, w.heads, w.heads, 128)
+    got = host.attention_fast_run(ctx, w.q[0], w.k[0], w.v[0], cfg, cpu=oracle_cpu)
+    want = zo.attention_run(w.q[0], w.k[0], w.v[0], oracle_cfg(cfg))
+    mx, mean = refimpl.check_close(got, want, "config1")
+    say(f"config1 max abs {mx:.2e} mean abs {mean:.2e}")
+    assert not np.array_equal(got, want)  # it really went through the bf16 kernel, not the CPU callback
+    again = host.attention_fast_run(ctx, w.q[0], w.k[0], w.v[0], cfg, cpu=None)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+
+
+# --------------------------------- configs 2-5, reduced size, every output row
+@pytest.mark.parametrize("name", ["klein_1024", "klein_512_x4", "zimage_1024", "klein_edit_ragged"])
+@pytest.mark.parametrize("k_site", [hip.K_IN_TILE_LOAD, hip.K_PREPASS])
+@pytest.mark.parametrize("dtype", [hip.BF16, hip.F32])
+def test_small_configs_all_rows(ctx, name, k_site, dtype):
+    say(f"small config {name} k_site={k_site} dtype={dtype}")
+    w = wl.by_name(name, seed=5, small=True)
+    res = wl.Resident(ctx, w, dtype=dtype, k_site=k_site)
+    got = res.run()
+    again = res.run()
+    res.release()
+    want = refimpl.reference_rows(w)
+    mx, mean = refimpl.check_close(got, want, name)
+    say(f"  S={w.tokens} H={w.heads} B={w.batch} max abs {mx:.2e} mean abs {mean:.2e}")
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+
+
+# ------------------------------------- configs 2-5, full size, sampled rows
+FULL = [("klein_1024", 48), ("klein_512_x4", 40), ("zimage_1024", 40), ("klein_edit_ragged", 28)]
+
+
+@pytest.mark.parametrize("name,nsample", FULL)
+def test_full_configs_sampled_rows_and_bit_stability(ctx, name, nsample):
+    say(f"full config {name}")
+    w = wl.by_name(name, seed=0)
+    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_IN_TILE_LOAD)
+    got = res.run()
+    say("  gpu done, checking stability")
+    for _ in range(3):
+        again = res.run()
+        assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), "output differs between runs"
+    res.k_site = hip.K_PREPASS
+    res.ext.k_site = hip.K_PREPASS
+    pre = res.run()
+    res.release()
+    toks = refimpl.sample_tokens(w, nsample)
+    say(f"  oracle on {len(toks)} query tokens x {w.batch} segments")
+    want = refimpl.reference_rows(w, toks)
+    mx, mean = refimpl.check_close(got[:, toks], want, name)
+    say(f"  tile-load K: max abs {mx:.2e} mean abs {mean:.2e}")
+    mx, mean = refimpl.check_close(pre[:, toks], want, name + " (K pre-pass)")
+    say(f"  pre-pass  K: max abs {mx:.2e} mean abs {mean:.2e}")
+    assert np.isfinite(got).all() and np.isfinite(pre).all()
+    # no row left unwritten: every output row has a non-zero element
+    assert (np.abs(got).max(axis=-1) > 0).all()
+
+
+# ----------------------------------------------------- size-independent properties
+def test_segments_are_independent(ctx):
+    # klein/zflux2_resident.zig:1803-1833: attention never crosses image segments
+    w = wl.by_name("klein_512_x4", seed=2, small=True)
+    res = wl.Resident(ctx, w)
+    full = res.run()
+    res.release()
+    for b in range(w.batch):
+        one = wl.klein(seed=0, batch=1, heads=w.heads, grid=w.grid, txt_len=w.txt_len, theta=w.theta)
+        one.q, one.k, one.v = w.q[b:b + 1], w.k[b:b + 1], w.v[b:b + 1]
+        r1 = wl.Resident(ctx, one)
+        single = r1.run()
+        r1.release()
+        assert np.array_equal(full[b].view(np.uint32), single[0].view(np.uint32))
+
+
+def test_key_padding_equals_deleting_the_keys(ctx):
+    # masked keys must not influence any row: replace them with huge values
+    w = wl.by_name("klein_edit_ragged", seed=4, small=True)
+    res = wl.Resident(ctx, w)
+    base = res.run()
+    res.release()
+    w2 = wl.by_name("klein_edit_ragged", seed=4, small=True)
+    for b in range(w2.batch):
+        m = w2.key_pad[b] != 0
+        w2.k[b, m] = 1e4
+        w2.v[b, m] = -7e4
+    res2 = wl.Resident(ctx, w2)
+    poisoned = res2.run()
+    res2.release()
+    # query rows at masked positions have different Q only if Q was changed; it was not
+    assert np.array_equal(base.view(np.uint32), poisoned.view(np.uint32))
+
+
+def test_text_row_weights_select_by_token(ctx):
+    # double blocks: text rows use norm_added_q/k, image rows norm_q/k
+    # (klein/zflux2_dit.zig:311-314). With distinct weights the result must equal
+    # the oracle's per-range normalisation.
+    w = wl.by_name("klein_1024", seed=6, small=True)
+    rng = np.random.default_rng(0)
+    wq, wk, wqt, wkt = (1.0 + 0.3 * rng.standard_normal(128).astype(np.float32) for _ in range(4))
+    q16 = host.f32_to_bf16_bits(w.q)
+    k16 = host.f32_to_bf16_bits(w.k)
+    v16 = host.f32_to_bf16_bits(w.v)
+    bufs = [ctx.buffer(a) for a in (q16, k16, v16)]
+    o = ctx.buffer(nbytes=q16.nbytes)
+    wb = [ctx.buffer(a) for a in (wq, wk, wqt, wkt)]
+    cos, sin = ctx.buffer(w.rope_cos), ctx.buffer(w.rope_sin)
+    ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=w.tokens, heads=w.heads, norm_q=wb[0], norm_k=wb[1],
+                    norm_added_q=wb[2], norm_added_k=wb[3], txt_rows=w.txt_len, rope_cos=cos, rope_sin=sin)
+    got = host.bf16_bits_to_f32(o.read(np.uint16, w.q.shape))[0]
+    t = w.txt_len
+    qn = np.concatenate([zo.klein_rms_norm_heads(w.q[0, :t], wqt), zo.klein_rms_norm_heads(w.q[0, t:], wq)])
+    kn = np.concatenate([zo.klein_rms_norm_heads(w.k[0, :t], wkt), zo.klein_rms_norm_heads(w.k[0, t:], wk)])
+    c2, s2 = zo.klein_build_rope_ref(w.grid[0], w.grid[1], theta=w.theta, txt_len=t)
+    qn, kn = zo.klein_apply_rope(qn, c2, s2), zo.klein_apply_rope(kn, c2, s2)
+    want = zo.attention_run(qn, kn, w.v[0], zo.Config(w.tokens, w.heads, w.heads, 128))
+    refimpl.check_close(got, want, "text-row weights")
+    for b in bufs + wb + [o, cos, sin]:
+        b.release()
+
+
+# ----------------------------------------------------------- C-ABI level behaviour
+def test_batch_offsets_address_image_segments(ctx):
+    # zdraw_metal_run_attention_enc_off: one call per segment at byte offsets
+    L = hip.lib()
+    rng = np.random.default_rng(8)
+    nb, tokens, heads = 3, 70, 2
+    q, k, v = (rng.standard_normal((nb, tokens, heads, 128), dtype=np.float32) for _ in range(3))
+    qb, kb, vb = ctx.buffer(q), ctx.buffer(k), ctx.buffer(v)
+    ob = ctx.buffer(nbytes=q.nbytes)
+    params = hip.AttnParams(tokens, heads, heads, 128, 0, 0)
+    batch = L.zdraw_hip_batch_begin(ctx.queue)
+    assert batch
+    seg = tokens * heads * 128 * 4
+    d0 = L.zdraw_hip_dispatch_count()
+    for i in range(nb):
+        rc = L.zdraw_hip_run_attention_enc_off(batch, ctx.block_pipeline, qb.handle, kb.handle, vb.handle, ob.handle,
+                                               C.byref(params), hip.K_BLOCK, 0, i * seg, i * seg)
+        assert rc == 0, hip.last_error()
+    assert L.zdraw_hip_batch_end(batch) == 0
+    assert L.zdraw_hip_dispatch_count() - d0 == nb
+    got = ob.read(np.float32, q.shape)
+    cfg = zo.Config(tokens, heads, heads, 128)
+    for i in range(nb):
+        refimpl.check_close(got[i], zo.attention_run(q[i], k[i], v[i], cfg), f"segment {i}")
+    # run_on_handles == the same kernel on caller-owned handles (mattn.zig:228-250)
+    o2 = ctx.buffer(nbytes=seg)
+    q0, k0, v0 = ctx.buffer(q[0]), ctx.buffer(k[0]), ctx.buffer(v[0])
+    ctx.run_on_handles(q0.handle, k0.handle, v0.handle, o2.handle, host.Config(tokens, heads, heads, 128))
+    assert np.array_equal(o2.read(np.float32, q[0].shape).view(np.uint32), got[0].view(np.uint32))
+    for b in (qb, kb, vb, ob, o2, q0, k0, v0):
+        b.release()
+
+
+def test_abi_return_codes(ctx):
+    L = hip.lib()
+    tokens, heads = 64, 2
+    n = tokens * heads * 128
+    buf = ctx.buffer(np.zeros(n, np.float32))
+    small = ctx.buffer(np.zeros(n - 128, np.float32))
+
+    def run(params, q=buf, kernel=hip.K_BLOCK):
+        return L.zdraw_hip_run_attention(ctx.queue, ctx.block_pipeline, q.handle, buf.handle, buf.handle, buf.handle,
+                                         C.byref(params), kernel, 0)
+
+    f0 = L.zdraw_hip_attn_fallback_count()
+    assert run(hip.AttnParams(tokens, heads, heads, 128, 0, 0)) == hip.OK
+    assert run(hip.AttnParams(tokens, heads, heads, 64, 0, 0)) == hip.UNAVAILABLE
+    assert run(hip.AttnParams(tokens, heads, heads, 128, 1, 0)) == hip.UNAVAILABLE
+    assert run(hip.AttnParams(tokens, heads, 1, 128, 0, 0)) == hip.UNAVAILABLE
+    assert run(hip.AttnParams(0, heads, heads, 128, 0, 0)) == hip.UNAVAILABLE
+    assert run(hip.AttnParams(tokens, heads, heads, 128, 0, 0), kernel=hip.K_ROWS) == hip.UNAVAILABLE
+    assert L.zdraw_hip_attn_fallback_count() - f0 == 5
+    assert run(hip.AttnParams(tokens, 0, heads, 128, 0, 0)) == hip.INVALID
+    assert run(hip.AttnParams(tokens, 3, 2, 128, 0, 0)) == hip.INVALID
+    assert run(hip.AttnParams(tokens, heads, heads, 128, 0, 0), q=small) == hip.INVALID
+    assert "too small" in hip.last_error()
+    assert L.zdraw_hip_run_attention(None, ctx.block_pipeline, buf.handle, buf.handle, buf.handle, buf.handle,
+                                     C.byref(hip.AttnParams(tokens, heads, heads, 128, 0, 0)), hip.K_BLOCK, 0) == hip.ERR_HANDLE
+    # misaligned offset in the fused entry
+    x = hip.AttnExt()
+    for s in (x.q_stride, x.k_stride, x.v_stride, x.out_stride):
+        s[0], s[1], s[2] = 0, heads * 128, 128
+    x.batch, x.in_dtype, x.out_dtype = 1, hip.F32, hip.F32
+    x.q_off = 4
+    p = hip.AttnParams(tokens - 1, heads, heads, 128, 0, 0)
+    rc = L.zdraw_hip_run_attention_fused(ctx.queue, buf.handle, buf.handle, buf.handle, buf.handle, C.byref(p),
+                                         C.byref(x), None)
+    assert rc == hip.INVALID
+    x.q_off = 0
+    x.qk_mode = hip.QK_KLEIN  # operands missing
+    rc = L.zdraw_hip_run_attention_fused(ctx.queue, buf.handle, buf.handle, buf.handle, buf.handle, C.byref(p),
+                                         C.byref(x), None)
+    assert rc == hip.INVALID
+    buf.release()
+    small.release()
+
+
+def test_scratch_is_grow_only_and_filled(ctx):
+    L = hip.lib()
+    a = L.zdraw_hip_attn_scratch(ctx.device, 4, 4096)
+    assert a and L.zdraw_hip_buffer_length(a) >= 4096
+    out = np.ones(4096, np.uint8)
+    L.zdraw_hip_read_buffer(a, out.ctypes.data_as(C.c_void_p), 4096)
+    assert not out.any()
+    b = L.zdraw_hip_attn_scratch(ctx.device, 4, 1024)
+    assert b == a and L.zdraw_hip_buffer_length(b) >= 4096
+    c = L.zdraw_hip_attn_scratch(ctx.device, 4, 1 << 20)
+    assert L.zdraw_hip_buffer_length(c) >= (1 << 20)
+    assert not L.zdraw_hip_attn_scratch(ctx.device, 5, 16)
+
+
+# --------------------------------------------- standalone QK-norm + rope (mqk.run)
+def test_qk_norm_rope_in_place_matches_oracle(ctx):
+    rng = np.random.default_rng(9)
+    tokens, heads = 77, 3
+    pos = np.stack([rng.integers(0, 1536, tokens), rng.integers(0, 512, tokens), rng.integers(0, 512, tokens)], 1)
+    q = rng.standard_normal((tokens, heads, 128), dtype=np.float32)
+    k = rng.standard_normal((tokens, heads, 128), dtype=np.float32)
+    qw = 1.0 + 0.2 * rng.standard_normal(128).astype(np.float32)
+    kw = 1.0 + 0.2 * rng.standard_normal(128).astype(np.float32)
+    cfg = zo.RopeConfig(wl.ZIMAGE_DIMS, wl.ZIMAGE_LENS, wl.ZIMAGE_THETA)
+    vals = zo.zrope_fill(cfg)
+    qb, kb = ctx.buffer(q), ctx.buffer(k)
+    ctx.qk_run(qb, kb, qw, kw, pos, vals, wl.ZIMAGE_DIMS, wl.ZIMAGE_LENS, tokens=tokens, heads=heads,
+               kv_heads=heads, head_dim=128, norm_eps=wl.ZIMAGE_EPS)
+    gq, gk = qb.read(np.float32, q.shape), kb.read(np.float32, k.shape)
+    wq_ref = zo.zimage_rotate(zo.zimage_norm_heads(q, qw, wl.ZIMAGE_EPS), vals, cfg, pos)
+    wk_ref = zo.zimage_rotate(zo.zimage_norm_heads(k, kw, wl.ZIMAGE_EPS), vals, cfg, pos)
+    # fp32 on both sides: only the summation order of the mean square and rsqrt differ
+    assert np.abs(gq - wq_ref).max() < 5e-6 * np.abs(wq_ref).max() + 2e-6
+    assert np.abs(gk - wk_ref).max() < 5e-6 * np.abs(wk_ref).max() + 2e-6
+    bad = pos.copy()
+    bad[5, 1] = 512
+    with pytest.raises(host.BadPosition):  # zrope.zig:48
+        ctx.qk_run(qb, kb, qw, kw, bad, vals, wl.ZIMAGE_DIMS, wl.ZIMAGE_LENS, tokens=tokens, heads=heads,
+                   kv_heads=heads, head_dim=128, norm_eps=wl.ZIMAGE_EPS)
+    qb.release()
+    kb.release()

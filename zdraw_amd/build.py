@@ -1,0 +1,71 @@
+"""Builds the gfx950 shared libraries in-tree with hipcc / g++.
+
+`python -m zdraw_amd.build` compiles
+  zdraw_amd/lib/libzdraw_hip.so   the C-ABI library (HIP kernels + bridge)
+  zdraw_amd/lib/libzdraw_host.so  the C++ host layer above the C ABI
+hipcc cross-compiles for gfx950 without a GPU present.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+HOST = os.path.join(HERE, "host")
+LIBDIR = os.path.join(HERE, "lib")
+
+HIP_LIB = os.path.join(LIBDIR, "libzdraw_hip.so")
+HOST_LIB = os.path.join(LIBDIR, "libzdraw_host.so")
+
+# Packed-FP32 VALU forms are disabled for every device translation unit.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stdout + proc.stderr)
+        raise RuntimeError("build failed: " + " ".join(cmd))
+    return proc
+
+
+def build_hip(verbose: bool = False) -> str:
+    os.makedirs(LIBDIR, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    srcs = [os.path.join(CSRC, "attn_kernel.hip"), os.path.join(CSRC, "bridge.hip")]
+    objs = []
+    for src in srcs:
+        obj = os.path.join(LIBDIR, os.path.basename(src) + ".o")
+        _run([hipcc, *HIPCC_FLAGS, "-c", src, "-o", obj])
+        objs.append(obj)
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB, *objs])
+    if verbose:
+        print("built", HIP_LIB)
+    return HIP_LIB
+
+
+def build_host(verbose: bool = False) -> str:
+    os.makedirs(LIBDIR, exist_ok=True)
+    srcs = [os.path.join(HOST, f) for f in sorted(os.listdir(HOST)) if f.endswith(".cc")]
+    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+          "-I", os.path.join(ROOT, "include"), "-o", HOST_LIB, *srcs,
+          "-L", LIBDIR, "-lzdraw_hip", "-Wl,-rpath,$ORIGIN"])
+    if verbose:
+        print("built", HOST_LIB)
+    return HOST_LIB
+
+
+def build_all(verbose: bool = False):
+    build_hip(verbose)
+    build_host(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)

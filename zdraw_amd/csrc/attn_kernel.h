@@ -1,0 +1,97 @@
+// Internal launch interface between the C-ABI bridge and the gfx950 kernels.
+// Not part of the public ABI (that is include/zdraw_hip.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace zdraw {
+
+constexpr int kHeadDim = 128;      // the only head width the MFMA kernel is built for
+constexpr int kKeyTile = 64;       // keys per LDS tile
+constexpr int kMaxKeyTiles = 4096; // key-tile list capacity in LDS (tokens <= 262144)
+
+enum QkMode : int {
+    kQkNone = 0,   // operands are used as given
+    kQkKlein = 1,  // RMSNorm(eps, learned weight) then table rope (cos/sin [rows][128])
+    kQkZimage = 2, // RMSNorm then 3-axis complex-pair rope from pos[rows][3] and a pair table
+};
+
+enum DType : int { kF32 = 0, kF16 = 1, kBF16 = 2 };
+
+// Side operands of the QK-norm + rope step, shared by the attention kernel
+// and the standalone pre-pass.
+struct QkOps {
+    // Klein rope table rows, [rows][128] f32; row = segment * rope_bs + token
+    const float* rope_cos;
+    const float* rope_sin;
+    // Z-Image: positions u64[rows][3] and (cos,sin) pair table
+    const unsigned long long* pos;
+    const float* pairs;
+    int64_t rope_bs;    // table / position rows between segments (0 = shared)
+    uint32_t base0, base1, base2; // Z-Image axis bases in pairs
+    int32_t dim0, dim1, dim2;     // Z-Image axis widths
+    int32_t txt_rows;   // tokens < txt_rows use the *_txt weights when given
+    float eps;
+};
+
+// Everything one attention launch needs, passed by value as the kernel argument.
+// Strides are in elements; the head_dim axis is contiguous.
+struct AttnArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    int64_t q_bs, q_ts, q_hs;
+    int64_t k_bs, k_ts, k_hs;
+    int64_t v_bs, v_ts, v_hs;
+    int64_t o_bs, o_ts, o_hs;
+    int32_t tokens;     // S: queries and keys per segment
+    int32_t heads;      // H
+    int32_t batch;      // independent segments
+    int32_t key_limit;  // keys >= key_limit are excluded (min(S, valid))
+    int32_t nqb;        // query blocks per (segment, head)
+    int32_t q_mode;     // QkMode applied to Q rows at load
+    int32_t out_dtype;  // kF32 or kBF16
+    float scale_log2;   // log2(e) / sqrt(head_dim)
+    QkOps qk;
+    // QK-norm weights (f32[128]); *_txt used for tokens < qk.txt_rows when non-null
+    const float* q_w;
+    const float* k_w;
+    const float* q_w_txt;
+    const float* k_w_txt;
+    // key-padding mask, u8 [segment][tokens], nonzero = key excluded; may be null
+    const unsigned char* key_pad;
+    int64_t mask_bs;    // bytes between segments (0 = shared)
+};
+
+// Standalone norm + rope over rows of one operand (Q or K): the pre-pass for
+// K and the in-place qk_norm_rope entry. Output may alias the input.
+struct PrepArgs {
+    const void* x;
+    void* y;
+    int64_t x_bs, x_ts, x_hs;
+    int64_t y_bs, y_ts, y_hs;
+    int32_t tokens, heads, batch;
+    int32_t mode;       // QkMode (never kQkNone)
+    int32_t out_dtype;  // kF32 or kBF16
+    int32_t pad0;
+    QkOps qk;
+    const float* w;
+    const float* w_txt;
+};
+
+// LDS bytes the attention kernel needs (dynamic shared memory).
+size_t attention_lds_bytes();
+// Query rows per workgroup for a wave count (4 or 8).
+int attention_block_rows(int nwaves);
+
+// Launch one attention forward. in_dtype is kF32 or kBF16; k_mode is the
+// QkMode applied to K rows inside the K-tile load. Returns a hipError_t.
+hipError_t launch_attention(const AttnArgs& args, int in_dtype, int k_mode, int nwaves,
+                            hipStream_t stream);
+hipError_t launch_qk_prepass(const PrepArgs& args, int in_dtype, hipStream_t stream);
+// One-time per-device setup (raises the dynamic LDS limit on every instantiation).
+hipError_t attention_setup();
+
+} // namespace zdraw

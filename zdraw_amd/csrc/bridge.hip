@@ -1,0 +1,728 @@
+// C-ABI bridge of the gfx950 attention backend (include/zdraw_hip.h).
+//
+// Replaces the attention slice of the reference's Objective-C Metal bridge
+// (metal/metal_api.m: device/queue/buffer lifecycle :536-576, standalone and
+// batch attention encode :2976-3125, scratch slots :6147-6191, the steel route
+// :6772-6815, batch begin/end :1084-1114, counters :333-353). Handles are
+// heap structs behind void*; every entry validates its operands on the host
+// before a kernel is launched, because a kernel that reads out of bounds can
+// take the whole device down.
+#include "../../include/zdraw_hip.h"
+#include "attn_kernel.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+using namespace zdraw;
+
+static_assert(sizeof(ZdrawAttnParams) == ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE, "AttnParams ABI drift");
+static_assert(sizeof(ZdrawHipAttnExt) == ZDRAW_HIP_ABI_ATTN_EXT_SIZE, "AttnExt ABI drift");
+static_assert(sizeof(ZdrawHipQkOperands) == ZDRAW_HIP_ABI_QK_OPERANDS_SIZE, "QkOperands ABI drift");
+
+namespace {
+
+struct Device {
+    int ordinal;
+};
+struct Queue {
+    Device* dev;
+    hipStream_t stream;
+};
+struct Buffer {
+    void* ptr;
+    size_t len;
+    bool owned;
+};
+struct Pipeline {
+    int kind; // 0 = attention_block_mfma, 1 = qk_norm_rope
+};
+struct Batch {
+    Queue* queue;
+    hipEvent_t start;
+    hipEvent_t stop;
+};
+struct Event {
+    hipEvent_t ev;
+};
+
+// Single-threaded counters, as in the reference bridge (metal_api.m:333-353).
+uint64_t g_dispatch = 0;
+uint64_t g_command = 0;
+uint64_t g_fallback = 0;
+uint64_t g_gpu_ns = 0;
+int g_waves = 8;
+bool g_setup_done = false;
+
+thread_local char g_err[512] = "";
+
+void set_err(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    set_err("%s: %s", what, hipGetErrorString(e));
+    return ZDRAW_HIP_ERR_DEVICE;
+}
+
+int unavailable(const char* why) {
+    g_fallback++;
+    set_err("unavailable: %s", why);
+    return ZDRAW_HIP_UNAVAILABLE;
+}
+
+int invalid(const char* why) {
+    set_err("invalid: %s", why);
+    return ZDRAW_HIP_INVALID;
+}
+
+size_t elem_size(uint32_t dtype) { return dtype == ZDRAW_HIP_F32 ? 4 : 2; }
+
+// One strided activation operand checked against its buffer.
+struct Operand {
+    const Buffer* buf;
+    uint64_t off;          // bytes
+    uint64_t bs, ts, hs;   // elements
+};
+
+// Returns nullptr if fine, else a reason. The kernel issues 16-byte loads of
+// 8 (bf16) or 4 (f32) consecutive elements, and 8/16-byte stores of 4.
+const char* check_operand(const Operand& o, uint32_t dtype, uint32_t batch, uint32_t tokens, uint32_t heads,
+                          const char* name) {
+    static thread_local char why[128];
+    if (!o.buf || !o.buf->ptr) {
+        snprintf(why, sizeof(why), "%s: null buffer", name);
+        return why;
+    }
+    const size_t es = elem_size(dtype);
+    const uint64_t align_elems = 16 / es;
+    if (o.off % 16 != 0 || o.ts % align_elems != 0 || o.hs % align_elems != 0 || (batch > 1 && o.bs % align_elems != 0)) {
+        snprintf(why, sizeof(why), "%s: offset/strides must keep rows 16-byte aligned", name);
+        return why;
+    }
+    if (((uintptr_t)o.buf->ptr) % 16 != 0) {
+        snprintf(why, sizeof(why), "%s: device pointer not 16-byte aligned", name);
+        return why;
+    }
+    if (o.ts < kHeadDim && tokens > 1) {
+        snprintf(why, sizeof(why), "%s: token stride smaller than head_dim", name);
+        return why;
+    }
+    const uint64_t last = (uint64_t)(batch - 1) * o.bs + (uint64_t)(tokens - 1) * o.ts + (uint64_t)(heads - 1) * o.hs +
+                          kHeadDim;
+    if (o.off > o.buf->len || last * es > o.buf->len - o.off) {
+        snprintf(why, sizeof(why), "%s: buffer too small for the declared shape", name);
+        return why;
+    }
+    return nullptr;
+}
+
+const void* at(const Buffer* b, uint64_t off) { return static_cast<const char*>(b->ptr) + off; }
+
+bool need(const void* handle, size_t bytes) {
+    const Buffer* b = static_cast<const Buffer*>(handle);
+    return b && b->ptr && b->len >= bytes && ((uintptr_t)b->ptr % 16) == 0;
+}
+
+struct FusedPlan {
+    AttnArgs args;
+    int in_dtype;
+    int k_mode;
+    bool prepass;
+    PrepArgs prep;
+};
+
+// Shared validation + argument assembly. Returns 0 or an ABI return code.
+int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const ZdrawAttnParams* p,
+                   const ZdrawHipAttnExt* x, const ZdrawHipQkOperands* ops, FusedPlan* plan) {
+    if (!p || !x) {
+        set_err("null params");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    // shape classes, in the order mattn.zig:376-408 checks them
+    if (p->tokens == 0) return unavailable("tokens == 0");
+    if (p->heads == 0 || p->kv_heads == 0 || p->head_dim == 0) return invalid("zero dimension");
+    if (p->heads % p->kv_heads != 0) return invalid("heads % kv_heads != 0");
+    if (p->head_dim != (uint32_t)kHeadDim) return unavailable("head_dim != 128");
+    if (p->causal != 0) return unavailable("causal attention");
+    if (p->kv_heads != p->heads) return unavailable("grouped-query attention");
+    if (x->batch == 0) return invalid("batch == 0");
+    if ((uint64_t)p->tokens > (uint64_t)kMaxKeyTiles * kKeyTile) return unavailable("too many tokens");
+    if ((x->in_dtype != ZDRAW_HIP_F32 && x->in_dtype != ZDRAW_HIP_BF16) ||
+        (x->out_dtype != ZDRAW_HIP_F32 && x->out_dtype != ZDRAW_HIP_BF16))
+        return unavailable("activation dtype");
+    if (x->qk_mode > ZDRAW_HIP_QK_ZIMAGE) return invalid("qk_mode");
+
+    const Operand oq{static_cast<Buffer*>(q), x->q_off, x->q_stride[0], x->q_stride[1], x->q_stride[2]};
+    const Operand ok{static_cast<Buffer*>(k), x->k_off, x->k_stride[0], x->k_stride[1], x->k_stride[2]};
+    const Operand ov{static_cast<Buffer*>(v), x->v_off, x->v_stride[0], x->v_stride[1], x->v_stride[2]};
+    const Operand oo{static_cast<Buffer*>(out), x->out_off, x->out_stride[0], x->out_stride[1], x->out_stride[2]};
+    const char* why;
+    if ((why = check_operand(oq, x->in_dtype, x->batch, p->tokens, p->heads, "q"))) return invalid(why);
+    if ((why = check_operand(ok, x->in_dtype, x->batch, p->tokens, p->heads, "k"))) return invalid(why);
+    if ((why = check_operand(ov, x->in_dtype, x->batch, p->tokens, p->heads, "v"))) return invalid(why);
+    if ((why = check_operand(oo, x->out_dtype, x->batch, p->tokens, p->heads, "out"))) return invalid(why);
+
+    AttnArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = at(oq.buf, oq.off);
+    a.k = at(ok.buf, ok.off);
+    a.v = at(ov.buf, ov.off);
+    a.o = const_cast<void*>(at(oo.buf, oo.off));
+    a.q_bs = (int64_t)oq.bs; a.q_ts = (int64_t)oq.ts; a.q_hs = (int64_t)oq.hs;
+    a.k_bs = (int64_t)ok.bs; a.k_ts = (int64_t)ok.ts; a.k_hs = (int64_t)ok.hs;
+    a.v_bs = (int64_t)ov.bs; a.v_ts = (int64_t)ov.ts; a.v_hs = (int64_t)ov.hs;
+    a.o_bs = (int64_t)oo.bs; a.o_ts = (int64_t)oo.ts; a.o_hs = (int64_t)oo.hs;
+    a.tokens = (int32_t)p->tokens;
+    a.heads = (int32_t)p->heads;
+    a.batch = (int32_t)x->batch;
+    a.key_limit = (int32_t)((p->valid != 0 && p->valid < p->tokens) ? p->valid : p->tokens);
+    const int rows = attention_block_rows(g_waves);
+    a.nqb = (int32_t)((p->tokens + rows - 1) / rows);
+    a.q_mode = (int32_t)x->qk_mode;
+    a.out_dtype = (int32_t)x->out_dtype;
+    a.scale_log2 = 1.4426950408889634f / sqrtf((float)kHeadDim);
+    if ((int64_t)a.nqb * a.heads * a.batch > 0x7fffffffLL) return unavailable("grid too large");
+
+    const uint64_t rows_needed = (uint64_t)(x->batch - 1) * x->rope_batch_rows + p->tokens;
+    if (x->qk_mode != ZDRAW_HIP_QK_NONE) {
+        if (!ops) return invalid("qk_mode set without operands");
+        if (!need(ops->q_weight, kHeadDim * 4) || !need(ops->k_weight, kHeadDim * 4))
+            return invalid("norm weights must be f32[128] buffers");
+        if ((ops->q_weight_txt && !need(ops->q_weight_txt, kHeadDim * 4)) ||
+            (ops->k_weight_txt && !need(ops->k_weight_txt, kHeadDim * 4)))
+            return invalid("text norm weights must be f32[128] buffers");
+        if (!(x->eps >= 0.0f)) return invalid("eps");
+        a.q_w = static_cast<const float*>(static_cast<Buffer*>(ops->q_weight)->ptr);
+        a.k_w = static_cast<const float*>(static_cast<Buffer*>(ops->k_weight)->ptr);
+        a.q_w_txt = ops->q_weight_txt ? static_cast<const float*>(static_cast<Buffer*>(ops->q_weight_txt)->ptr) : nullptr;
+        a.k_w_txt = ops->k_weight_txt ? static_cast<const float*>(static_cast<Buffer*>(ops->k_weight_txt)->ptr) : nullptr;
+        a.qk.txt_rows = (int32_t)x->txt_rows;
+        a.qk.eps = x->eps;
+        a.qk.rope_bs = (int64_t)x->rope_batch_rows;
+        if (x->qk_mode == ZDRAW_HIP_QK_KLEIN) {
+            const size_t bytes = (size_t)rows_needed * kHeadDim * 4;
+            if (!need(ops->rope_cos, bytes) || !need(ops->rope_sin, bytes))
+                return invalid("rope cos/sin tables too small for [rows][128] f32");
+            a.qk.rope_cos = static_cast<const float*>(static_cast<Buffer*>(ops->rope_cos)->ptr);
+            a.qk.rope_sin = static_cast<const float*>(static_cast<Buffer*>(ops->rope_sin)->ptr);
+        } else {
+            const uint32_t* d = x->zimage_dims;
+            if (d[0] + d[1] + d[2] != (uint32_t)kHeadDim) return invalid("zimage dims must sum to head_dim");
+            if (d[0] % 8 != 0 || d[1] % 8 != 0 || d[2] % 8 != 0 || d[0] == 0 || d[1] == 0 || d[2] == 0)
+                return unavailable("zimage axis widths must be non-zero multiples of 8");
+            for (int i = 0; i < 3; i++)
+                if (x->zimage_base[i] % 2 != 0 || x->zimage_base[i] > 0xffffffffull)
+                    return unavailable("zimage axis bases must be even and fit 32 bits");
+            if (!need(ops->pos, (size_t)rows_needed * 24)) return invalid("positions too small for [rows][3] u64");
+            if (!need(ops->rope_pairs, 16)) return invalid("rope pair table missing");
+            // every axis must have at least one position's worth of pairs inside the table
+            const Buffer* pt = static_cast<Buffer*>(ops->rope_pairs);
+            for (int i = 0; i < 3; i++)
+                if ((x->zimage_base[i] + d[i] / 2) * 8 > pt->len) return invalid("rope pair table smaller than an axis base");
+            a.qk.pos = static_cast<const unsigned long long*>(static_cast<Buffer*>(ops->pos)->ptr);
+            a.qk.pairs = static_cast<const float*>(pt->ptr);
+            a.qk.dim0 = (int32_t)d[0]; a.qk.dim1 = (int32_t)d[1]; a.qk.dim2 = (int32_t)d[2];
+            a.qk.base0 = (uint32_t)x->zimage_base[0];
+            a.qk.base1 = (uint32_t)x->zimage_base[1];
+            a.qk.base2 = (uint32_t)x->zimage_base[2];
+        }
+    }
+    if (ops && ops->key_pad) {
+        const Buffer* m = static_cast<Buffer*>(ops->key_pad);
+        const uint64_t mbytes = (uint64_t)(x->batch - 1) * x->mask_batch_bytes + p->tokens;
+        if (!m->ptr || m->len < mbytes) return invalid("key_pad smaller than [segments][tokens]");
+        a.key_pad = static_cast<const unsigned char*>(m->ptr);
+        a.mask_bs = (int64_t)x->mask_batch_bytes;
+    }
+
+    plan->args = a;
+    plan->in_dtype = (int)x->in_dtype;
+    plan->k_mode = (int)x->qk_mode;
+    plan->prepass = false;
+    if (x->qk_mode != ZDRAW_HIP_QK_NONE && x->k_site == ZDRAW_HIP_K_PREPASS) {
+        // K is normalised and rotated once into scratch slot 1, head-major, in
+        // the activation dtype; the attention kernel then reads it as is.
+        const size_t es = elem_size(x->in_dtype);
+        const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * es;
+        Buffer* s = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 1, bytes));
+        if (!s) {
+            set_err("scratch allocation failed");
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        PrepArgs pr;
+        memset(&pr, 0, sizeof(pr));
+        pr.x = a.k;
+        pr.y = s->ptr;
+        pr.x_bs = a.k_bs; pr.x_ts = a.k_ts; pr.x_hs = a.k_hs;
+        pr.y_bs = (int64_t)p->heads * p->tokens * kHeadDim;
+        pr.y_ts = kHeadDim;
+        pr.y_hs = (int64_t)p->tokens * kHeadDim;
+        pr.tokens = a.tokens; pr.heads = a.heads; pr.batch = a.batch;
+        pr.mode = (int32_t)x->qk_mode;
+        pr.out_dtype = (int32_t)x->in_dtype;
+        pr.qk = a.qk;
+        pr.w = a.k_w;
+        pr.w_txt = a.k_w_txt;
+        plan->prep = pr;
+        plan->prepass = true;
+        plan->k_mode = kQkNone;
+        plan->args.k = s->ptr;
+        plan->args.k_bs = pr.y_bs; plan->args.k_ts = pr.y_ts; plan->args.k_hs = pr.y_hs;
+    }
+    return ZDRAW_HIP_OK;
+}
+
+int enqueue(const FusedPlan& plan, hipStream_t stream) {
+    if (!g_setup_done) {
+        hipError_t e = attention_setup();
+        if (e != hipSuccess) {
+            set_err("attention_setup: %s", hipGetErrorString(e));
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        g_setup_done = true;
+    }
+    if (plan.prepass) {
+        hipError_t e = launch_qk_prepass(plan.prep, plan.in_dtype, stream);
+        if (e != hipSuccess) {
+            set_err("qk pre-pass launch: %s", hipGetErrorString(e));
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        g_dispatch++;
+    }
+    hipError_t e = launch_attention(plan.args, plan.in_dtype, plan.k_mode, g_waves, stream);
+    if (e != hipSuccess) {
+        set_err("attention launch: %s", hipGetErrorString(e));
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    g_dispatch++;
+    return ZDRAW_HIP_OK;
+}
+
+// Token-major f32 [tokens][heads][128] operands of the reference's standalone
+// entry (runtime/attention.zig:100-113), one segment at byte offsets.
+void standalone_ext(const ZdrawAttnParams* p, uint64_t in_off, uint64_t out_off, ZdrawHipAttnExt* x) {
+    memset(x, 0, sizeof(*x));
+    x->q_off = x->k_off = x->v_off = in_off;
+    x->out_off = out_off;
+    const uint64_t ts = (uint64_t)p->heads * p->head_dim;
+    uint64_t* strides[4] = {x->q_stride, x->k_stride, x->v_stride, x->out_stride};
+    for (auto* s : strides) {
+        s[0] = 0;
+        s[1] = ts;
+        s[2] = p->head_dim;
+    }
+    x->batch = 1;
+    x->in_dtype = ZDRAW_HIP_F32;
+    x->out_dtype = ZDRAW_HIP_F32;
+    x->qk_mode = ZDRAW_HIP_QK_NONE;
+}
+
+int check_pipeline(void* pipeline, uint32_t kernel, int want_kind) {
+    Pipeline* pl = static_cast<Pipeline*>(pipeline);
+    if (!pl) {
+        set_err("null pipeline");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    if (pl->kind != want_kind) {
+        set_err("pipeline of the wrong kind");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    if (want_kind == 0 && kernel != ZDRAW_HIP_K_BLOCK) return unavailable("only the block (MFMA) kernel exists");
+    return ZDRAW_HIP_OK;
+}
+
+int finish_blocking(Queue* qu, hipEvent_t start, hipEvent_t stop) {
+    hipError_t e = hipEventRecord(stop, qu->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(stop);
+    if (e != hipSuccess) return hip_fail(e, "wait");
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, start, stop) == hipSuccess && ms > 0.f) g_gpu_ns += (uint64_t)((double)ms * 1e6);
+    g_command++;
+    return ZDRAW_HIP_OK;
+}
+
+Buffer* g_scratch[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+
+bool scratch_poisoned(int slot) {
+    // ZDRAW_SCRATCH_POISON: "1" every slot, "attn" the group, "attn:2" one slot
+    const char* raw = getenv("ZDRAW_SCRATCH_POISON");
+    if (!raw || !*raw) return false;
+    if (strcmp(raw, "1") == 0) return true;
+    if (strncmp(raw, "attn", 4) != 0) return false;
+    if (raw[4] == '\0') return true;
+    if (raw[4] == ':') return atoi(raw + 5) == slot;
+    return false;
+}
+
+} // namespace
+
+extern "C" {
+
+// ---------------------------------------------------------------- lifecycle
+void* zdraw_hip_create_device(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        set_err("no HIP device");
+        return nullptr;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess) {
+        set_err("hipGetDeviceProperties failed");
+        return nullptr;
+    }
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_err("device 0 is %s; this library is built for gfx950 only", prop.gcnArchName);
+        return nullptr;
+    }
+    if (hipSetDevice(0) != hipSuccess) return nullptr;
+    Device* d = new Device{0};
+    return d;
+}
+
+void zdraw_hip_release_device(void* device) { delete static_cast<Device*>(device); }
+
+void* zdraw_hip_create_queue(void* device) {
+    Device* d = static_cast<Device*>(device);
+    if (!d) return nullptr;
+    hipStream_t s;
+    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) {
+        set_err("hipStreamCreate failed");
+        return nullptr;
+    }
+    return new Queue{d, s};
+}
+
+void zdraw_hip_release_queue(void* queue) {
+    Queue* q = static_cast<Queue*>(queue);
+    if (!q) return;
+    (void)hipStreamSynchronize(q->stream);
+    (void)hipStreamDestroy(q->stream);
+    delete q;
+}
+
+// ------------------------------------------------------------------ buffers
+void* zdraw_hip_create_buffer(void* device, size_t size) {
+    if (!device || size == 0) return nullptr;
+    void* p = nullptr;
+    if (hipMalloc(&p, size) != hipSuccess) {
+        set_err("hipMalloc(%zu) failed", size);
+        return nullptr;
+    }
+    return new Buffer{p, size, true};
+}
+
+void* zdraw_hip_create_buffer_with_data(void* device, const uint8_t* data, size_t size) {
+    if (!data) return nullptr;
+    Buffer* b = static_cast<Buffer*>(zdraw_hip_create_buffer(device, size));
+    if (!b) return nullptr;
+    if (hipMemcpy(b->ptr, data, size, hipMemcpyHostToDevice) != hipSuccess) {
+        zdraw_hip_release_buffer(b);
+        set_err("upload failed");
+        return nullptr;
+    }
+    return b;
+}
+
+void* zdraw_hip_create_buffer_no_copy(void* device, void* device_ptr, size_t size) {
+    if (!device || !device_ptr || size == 0) return nullptr;
+    return new Buffer{device_ptr, size, false};
+}
+
+void zdraw_hip_read_buffer(void* buffer, uint8_t* dst, size_t size) {
+    Buffer* b = static_cast<Buffer*>(buffer);
+    if (!b || !dst || size > b->len) return;
+    (void)hipMemcpy(dst, b->ptr, size, hipMemcpyDeviceToHost);
+}
+
+void zdraw_hip_write_buffer(void* buffer, const uint8_t* src, size_t size) {
+    Buffer* b = static_cast<Buffer*>(buffer);
+    if (!b || !src || size > b->len) return;
+    (void)hipMemcpy(b->ptr, src, size, hipMemcpyHostToDevice);
+}
+
+size_t zdraw_hip_buffer_length(void* buffer) {
+    Buffer* b = static_cast<Buffer*>(buffer);
+    return b ? b->len : 0;
+}
+
+void* zdraw_hip_buffer_device_ptr(void* buffer) {
+    Buffer* b = static_cast<Buffer*>(buffer);
+    return b ? b->ptr : nullptr;
+}
+
+void zdraw_hip_release_buffer(void* buffer) {
+    Buffer* b = static_cast<Buffer*>(buffer);
+    if (!b) return;
+    if (b->owned && b->ptr) (void)hipFree(b->ptr);
+    delete b;
+}
+
+// ---------------------------------------------------------------- pipelines
+void* zdraw_hip_compile(void* device, const char* entry, char* error_buf, size_t error_len) {
+    if (error_buf && error_len) error_buf[0] = '\0';
+    if (!device || !entry) return nullptr;
+    if (strcmp(entry, "attention_block_mfma") == 0) return new Pipeline{0};
+    if (strcmp(entry, "qk_norm_rope") == 0) return new Pipeline{1};
+    if (error_buf && error_len) snprintf(error_buf, error_len, "no gfx950 kernel named '%s'", entry);
+    return nullptr;
+}
+
+void zdraw_hip_release_pipeline(void* pipeline) { delete static_cast<Pipeline*>(pipeline); }
+
+size_t zdraw_hip_pipeline_threads(void* pipeline) {
+    Pipeline* p = static_cast<Pipeline*>(pipeline);
+    if (!p) return 0;
+    return p->kind == 0 ? (size_t)g_waves * 64 : 256;
+}
+
+// ---------------------------------------------------------------- attention
+int zdraw_hip_run_attention(void* queue, void* pipeline, void* q, void* k, void* v, void* output,
+                            const ZdrawAttnParams* params, uint32_t kernel, size_t thread_count) {
+    (void)thread_count;
+    Queue* qu = static_cast<Queue*>(queue);
+    if (!qu || !params) {
+        set_err("null queue or params");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    int rc = check_pipeline(pipeline, kernel, 0);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    ZdrawHipAttnExt x;
+    standalone_ext(params, 0, 0, &x);
+    FusedPlan plan;
+    rc = plan_attention(qu->dev, q, k, v, output, params, &x, nullptr, &plan);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    hipEvent_t start, stop;
+    if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return ZDRAW_HIP_ERR_HANDLE;
+    (void)hipEventRecord(start, qu->stream);
+    rc = enqueue(plan, qu->stream);
+    if (rc == ZDRAW_HIP_OK) rc = finish_blocking(qu, start, stop);
+    (void)hipEventDestroy(start);
+    (void)hipEventDestroy(stop);
+    return rc;
+}
+
+void* zdraw_hip_batch_begin(void* queue) {
+    Queue* qu = static_cast<Queue*>(queue);
+    if (!qu) return nullptr;
+    Batch* b = new Batch{qu, nullptr, nullptr};
+    if (hipEventCreate(&b->start) != hipSuccess || hipEventCreate(&b->stop) != hipSuccess ||
+        hipEventRecord(b->start, qu->stream) != hipSuccess) {
+        delete b;
+        return nullptr;
+    }
+    return b;
+}
+
+int zdraw_hip_run_attention_enc_off(void* batch, void* pipeline, void* q, void* k, void* v, void* o,
+                                    const ZdrawAttnParams* params, uint32_t kernel, size_t thread_count,
+                                    uint64_t in_off, uint64_t out_off) {
+    (void)thread_count;
+    Batch* b = static_cast<Batch*>(batch);
+    if (!b || !params) {
+        set_err("null batch or params");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    int rc = check_pipeline(pipeline, kernel, 0);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    ZdrawHipAttnExt x;
+    standalone_ext(params, in_off, out_off, &x);
+    FusedPlan plan;
+    rc = plan_attention(b->queue->dev, q, k, v, o, params, &x, nullptr, &plan);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    return enqueue(plan, b->queue->stream);
+}
+
+int zdraw_hip_run_attention_enc(void* batch, void* pipeline, void* q, void* k, void* v, void* o,
+                                const ZdrawAttnParams* params, uint32_t kernel, size_t thread_count) {
+    return zdraw_hip_run_attention_enc_off(batch, pipeline, q, k, v, o, params, kernel, thread_count, 0, 0);
+}
+
+int zdraw_hip_batch_end(void* batch) {
+    Batch* b = static_cast<Batch*>(batch);
+    if (!b) return ZDRAW_HIP_ERR_HANDLE;
+    int rc = finish_blocking(b->queue, b->start, b->stop);
+    (void)hipEventDestroy(b->start);
+    (void)hipEventDestroy(b->stop);
+    delete b;
+    return rc;
+}
+
+int zdraw_hip_run_attention_fused_enc(void* batch, void* q, void* k, void* v, void* out,
+                                      const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                                      const ZdrawHipQkOperands* ops) {
+    Batch* b = static_cast<Batch*>(batch);
+    if (!b) {
+        set_err("null batch");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    FusedPlan plan;
+    int rc = plan_attention(b->queue->dev, q, k, v, out, params, ext, ops, &plan);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    return enqueue(plan, b->queue->stream);
+}
+
+int zdraw_hip_run_attention_fused(void* queue, void* q, void* k, void* v, void* out,
+                                  const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                                  const ZdrawHipQkOperands* ops) {
+    void* b = zdraw_hip_batch_begin(queue);
+    if (!b) {
+        set_err("null queue");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    int rc = zdraw_hip_run_attention_fused_enc(b, q, k, v, out, params, ext, ops);
+    int rc2 = zdraw_hip_batch_end(b);
+    return rc != ZDRAW_HIP_OK ? rc : rc2;
+}
+
+int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
+                               const ZdrawAttnParams* p, const ZdrawHipAttnExt* x,
+                               const ZdrawHipQkOperands* ops) {
+    Queue* qu = static_cast<Queue*>(queue);
+    if (!qu || !p || !x || !ops) {
+        set_err("null argument");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    int rc = check_pipeline(pipeline, 0, 1);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    if (p->tokens == 0) return unavailable("tokens == 0");
+    if (p->heads == 0 || p->kv_heads == 0) return invalid("zero dimension");
+    if (p->head_dim != (uint32_t)kHeadDim) return unavailable("head_dim != 128");
+    if (x->qk_mode != ZDRAW_HIP_QK_KLEIN && x->qk_mode != ZDRAW_HIP_QK_ZIMAGE) return invalid("qk_mode");
+    // Reuse the attention planner's operand validation by planning a
+    // same-shape launch over q (then k); nothing is enqueued from the plan
+    // except the pre-pass arguments assembled below.
+    ZdrawHipAttnExt sx;
+    for (int which = 0; which < 2; which++) {
+        ZdrawAttnParams sp = *p;
+        sp.heads = sp.kv_heads = which == 0 ? p->heads : p->kv_heads;
+        sp.causal = 0;
+        sp.valid = 0;
+        standalone_ext(&sp, 0, 0, &sx);
+        sx.qk_mode = x->qk_mode;
+        sx.eps = x->eps;
+        sx.txt_rows = x->txt_rows;
+        sx.rope_batch_rows = x->rope_batch_rows;
+        memcpy(sx.zimage_dims, x->zimage_dims, sizeof(sx.zimage_dims));
+        memcpy(sx.zimage_base, x->zimage_base, sizeof(sx.zimage_base));
+        void* buf = which == 0 ? q : k;
+        FusedPlan plan;
+        rc = plan_attention(qu->dev, buf, buf, buf, buf, &sp, &sx, ops, &plan);
+        if (rc != ZDRAW_HIP_OK) return rc;
+        PrepArgs pr;
+        memset(&pr, 0, sizeof(pr));
+        const AttnArgs& a = plan.args;
+        pr.x = a.q;
+        pr.y = a.o;
+        pr.x_bs = a.q_bs; pr.x_ts = a.q_ts; pr.x_hs = a.q_hs;
+        pr.y_bs = a.o_bs; pr.y_ts = a.o_ts; pr.y_hs = a.o_hs;
+        pr.tokens = a.tokens; pr.heads = a.heads; pr.batch = 1;
+        pr.mode = (int32_t)x->qk_mode;
+        pr.out_dtype = kF32;
+        pr.qk = a.qk;
+        pr.w = which == 0 ? a.q_w : a.k_w;
+        pr.w_txt = which == 0 ? a.q_w_txt : a.k_w_txt;
+        hipError_t e = launch_qk_prepass(pr, kF32, qu->stream);
+        if (e != hipSuccess) {
+            set_err("qk_norm_rope launch: %s", hipGetErrorString(e));
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        g_dispatch++;
+    }
+    hipError_t e = hipStreamSynchronize(qu->stream);
+    if (e != hipSuccess) return hip_fail(e, "qk_norm_rope wait");
+    g_command++;
+    return ZDRAW_HIP_OK;
+}
+
+// ------------------------------------------------------------------ scratch
+void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes) {
+    if (!device || slot < 0 || slot >= 5 || bytes == 0) return nullptr;
+    Buffer* cur = g_scratch[slot];
+    if (cur && cur->len >= bytes) return cur;
+    // Grow: work already enqueued may still read the old allocation, so drain
+    // the device before it is freed.
+    (void)hipDeviceSynchronize();
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        set_err("scratch hipMalloc(%zu) failed", bytes);
+        return nullptr;
+    }
+    // Filled at (re)allocation so a read that precedes its write sees the same
+    // bytes on every run (metal_api.m:6160-6181).
+    (void)hipMemset(p, scratch_poisoned(slot) ? 0xFF : 0x00, bytes);
+    (void)hipDeviceSynchronize();
+    if (cur) {
+        (void)hipFree(cur->ptr);
+        cur->ptr = p;
+        cur->len = bytes;
+        return cur;
+    }
+    g_scratch[slot] = new Buffer{p, bytes, true};
+    return g_scratch[slot];
+}
+
+// --------------------------------------------------------- counters, timing
+void zdraw_hip_metrics_reset(void) { g_dispatch = g_command = g_fallback = g_gpu_ns = 0; }
+uint64_t zdraw_hip_dispatch_count(void) { return g_dispatch; }
+uint64_t zdraw_hip_command_count(void) { return g_command; }
+uint64_t zdraw_hip_attn_fallback_count(void) { return g_fallback; }
+uint64_t zdraw_hip_gpu_ns(void) { return g_gpu_ns; }
+
+void* zdraw_hip_event_create(void) {
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return new Event{e};
+}
+int zdraw_hip_event_record(void* event, void* queue) {
+    Event* e = static_cast<Event*>(event);
+    Queue* q = static_cast<Queue*>(queue);
+    if (!e || !q) return ZDRAW_HIP_ERR_HANDLE;
+    return hipEventRecord(e->ev, q->stream) == hipSuccess ? ZDRAW_HIP_OK : ZDRAW_HIP_ERR_DEVICE;
+}
+int zdraw_hip_event_sync(void* event) {
+    Event* e = static_cast<Event*>(event);
+    if (!e) return ZDRAW_HIP_ERR_HANDLE;
+    return hipEventSynchronize(e->ev) == hipSuccess ? ZDRAW_HIP_OK : ZDRAW_HIP_ERR_DEVICE;
+}
+float zdraw_hip_event_elapsed_ms(void* start, void* stop) {
+    Event* a = static_cast<Event*>(start);
+    Event* b = static_cast<Event*>(stop);
+    float ms = -1.f;
+    if (!a || !b || hipEventElapsedTime(&ms, a->ev, b->ev) != hipSuccess) return -1.f;
+    return ms;
+}
+void zdraw_hip_event_release(void* event) {
+    Event* e = static_cast<Event*>(event);
+    if (!e) return;
+    (void)hipEventDestroy(e->ev);
+    delete e;
+}
+int zdraw_hip_queue_sync(void* queue) {
+    Queue* q = static_cast<Queue*>(queue);
+    if (!q) return ZDRAW_HIP_ERR_HANDLE;
+    hipError_t e = hipStreamSynchronize(q->stream);
+    return e == hipSuccess ? ZDRAW_HIP_OK : hip_fail(e, "queue sync");
+}
+
+void zdraw_hip_set_attention_waves(int nwaves) { g_waves = (nwaves == 4) ? 4 : 8; }
+
+size_t zdraw_hip_abi_sizeof(int which) {
+    switch (which) {
+    case 0: return sizeof(ZdrawAttnParams);
+    case 1: return sizeof(ZdrawHipAttnExt);
+    case 2: return sizeof(ZdrawHipQkOperands);
+    default: return 0;
+    }
+}
+
+const char* zdraw_hip_last_error(void) { return g_err; }
+
+} // extern "C"
