@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="klein_1024")
     ap.add_argument("--k-site", choices=["tile", "prepass"], default=os.environ.get("ZDRAW_BENCH_K_SITE", "tile"))
-    ap.add_argument("--waves", type=int, default=0)
+    ap.add_argument("--variant", type=int, default=0, help="kernel build: 0 default, 1/2 the 32-row kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -76,8 +76,7 @@ def main():
 
     L = hip.lib()
     ctx = host.Context.init()
-    if args.waves:
-        L.zdraw_hip_set_attention_waves(args.waves)
+    L.zdraw_hip_set_attention_variant(args.variant)
     w = wl.by_name(args.workload, seed=0)
     k_site = hip.K_PREPASS if args.k_site == "prepass" else hip.K_IN_TILE_LOAD
     res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=k_site)
@@ -139,7 +138,7 @@ def main():
         "config": {
             "workload": desc,
             "k_norm_rope_site": args.k_site,
-            "waves_per_workgroup": int(L.zdraw_hip_pipeline_threads(ctx.block_pipeline) // 64),
+            "kernel_variant": args.variant,
             "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
         },
         "roofline": {

@@ -194,8 +194,11 @@ float zdraw_hip_event_elapsed_ms(void* start, void* stop); /* negative on error 
 void zdraw_hip_event_release(void* event);
 int zdraw_hip_queue_sync(void* queue);
 
-/* Tuning knob for measurements: waves per workgroup (4 or 8; 0 = default). */
-void zdraw_hip_set_attention_waves(int nwaves);
+/* Measurement knob: which build of the attention kernel runs.
+ * Software-pipelined kernel: 0 = 64 query rows per wave x 4 waves (default),
+ * 1 = 32 rows x 8 waves, 2 = 32 rows x 4 waves (two workgroups per CU).
+ * Unpipelined kernel: 3 = 32 rows x 8 waves, 4 = 32 rows x 4 waves. */
+void zdraw_hip_set_attention_variant(int variant);
 
 /* ABI drift guard (src/abi_gen.zig, runtime/abi_assert.zig:29): sizeof of the
  * shared structs as this library was compiled. which: 0 = ZdrawAttnParams,

@@ -36,19 +36,23 @@ def _run(cmd):
     return proc
 
 
-def build_hip(verbose: bool = False) -> str:
+def build_hip(verbose: bool = False, out: str | None = None, extra_flags=()) -> str:
+    """Compile the C-ABI library. `out` / `extra_flags` build an experimental
+    copy elsewhere (kernel tuning defines) without touching the shipped one."""
     os.makedirs(LIBDIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(CSRC, "attn_kernel.hip"), os.path.join(CSRC, "bridge.hip")]
+    target = out or HIP_LIB
+    tag = "" if out is None else "." + os.path.basename(out)
+    srcs = [os.path.join(CSRC, f) for f in ("attn_kernel.hip", "attn_kernel_v2.hip", "bridge.hip")]
     objs = []
     for src in srcs:
-        obj = os.path.join(LIBDIR, os.path.basename(src) + ".o")
-        _run([hipcc, *HIPCC_FLAGS, "-c", src, "-o", obj])
+        obj = os.path.join(LIBDIR, os.path.basename(src) + tag + ".o")
+        _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-c", src, "-o", obj])
         objs.append(obj)
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB, *objs])
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", target, *objs])
     if verbose:
-        print("built", HIP_LIB)
-    return HIP_LIB
+        print("built", target)
+    return target
 
 
 def build_host(verbose: bool = False) -> str:

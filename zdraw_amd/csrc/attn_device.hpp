@@ -1,0 +1,204 @@
+// Device-side helpers shared by the gfx950 attention kernels: vector types,
+// global-memory chunk loads, bf16 packing, lane-pair reductions and the
+// QK-norm + rope arithmetic.
+#pragma once
+
+#include "attn_kernel.h"
+
+#include <type_traits>
+
+namespace zdraw {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int D = kHeadDim;
+
+// ---------------------------------------------------------------- raw loads
+// Eight consecutive head_dim elements as they come from memory.
+template <typename T> struct Raw8;
+template <> struct Raw8<float> { f32x4 a, b; };
+template <> struct Raw8<bf16_t> { u32x4 r; };
+
+template <typename T>
+__device__ __forceinline__ Raw8<T> ld_raw8(const T* p, bool ok) {
+    Raw8<T> x;
+    if constexpr (std::is_same<T, float>::value) {
+        x.a = f32x4{0.f, 0.f, 0.f, 0.f};
+        x.b = x.a;
+        if (ok) {
+            x.a = *reinterpret_cast<const f32x4*>(p);
+            x.b = *reinterpret_cast<const f32x4*>(p + 4);
+        }
+    } else {
+        x.r = u32x4{0u, 0u, 0u, 0u};
+        if (ok) x.r = *reinterpret_cast<const u32x4*>(p);
+    }
+    return x;
+}
+
+__device__ __forceinline__ void unpack8(const Raw8<float>& r, float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) { x[i] = r.a[i]; x[4 + i] = r.b[i]; }
+}
+__device__ __forceinline__ void unpack8(const Raw8<bf16_t>& r, float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        x[2 * i] = __uint_as_float(r.r[i] << 16);
+        x[2 * i + 1] = __uint_as_float(r.r[i] & 0xffff0000u);
+    }
+}
+
+// fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ u32x4 pack_bf16x8(const float (&x)[8]) {
+    f32x8 v;
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = x[i];
+    bf16x8 b = __builtin_convertvector(v, bf16x8);
+    return __builtin_bit_cast(u32x4, b);
+}
+__device__ __forceinline__ u32x4 raw_to_bf16(const Raw8<bf16_t>& r) { return r.r; }
+__device__ __forceinline__ u32x4 raw_to_bf16(const Raw8<float>& r) {
+    float x[8];
+    unpack8(r, x);
+    return pack_bf16x8(x);
+}
+
+// Two consecutive elements of one V row as a packed bf16 pair.
+__device__ __forceinline__ unsigned ld_pair_bf16(const bf16_t* p, bool ok) {
+    return ok ? *reinterpret_cast<const unsigned*>(p) : 0u;
+}
+__device__ __forceinline__ unsigned ld_pair_bf16(const float* p, bool ok) {
+    float x0 = 0.f, x1 = 0.f;
+    if (ok) {
+        const float2 t = *reinterpret_cast<const float2*>(p);
+        x0 = t.x;
+        x1 = t.y;
+    }
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    f32x2 v = {x0, x1};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+}
+
+// v_permlane32_swap with both operands = x returns, on every lane, the values
+// held by lane (l % 32) and lane (l % 32) + 32: the two lanes that share a query.
+__device__ __forceinline__ float pair_max(float x) {
+    u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+    u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// ------------------------------------------------------- QK-norm + rope math
+// Rope/weight operands for one row; `row` indexes the rope table / positions,
+// `tok` is the token index inside its segment (selects the text-row weights).
+struct QkRow {
+    const float* w;      // 128 weights for this row
+    const float* cos_r;  // Klein: table row
+    const float* sin_r;
+    unsigned long long p0, p1, p2; // Z-Image position
+};
+
+__device__ __forceinline__ QkRow qk_row(const QkOps& a, int mode, const float* w, const float* wt, int seg, int tok,
+                                        bool ok) {
+    QkRow r;
+    r.w = (wt != nullptr && tok < a.txt_rows) ? wt : w;
+    r.cos_r = r.sin_r = nullptr;
+    r.p0 = r.p1 = r.p2 = 0;
+    if (mode == kQkKlein) {
+        const int64_t row = ok ? (int64_t)seg * a.rope_bs + tok : 0;
+        r.cos_r = a.rope_cos + row * D;
+        r.sin_r = a.rope_sin + row * D;
+    } else if (mode == kQkZimage) {
+        const int64_t row = ok ? (int64_t)seg * a.rope_bs + tok : 0;
+        const unsigned long long* p = a.pos + row * 3;
+        r.p0 = p[0];
+        r.p1 = p[1];
+        r.p2 = p[2];
+    }
+    return r;
+}
+
+// Rope coefficients for the 8 elements starting at d0 (d0 % 8 == 0):
+// Klein: c[i], s[i] straight from the table row (klein/zflux2_dit.zig:213-228
+// reads both columns of a pair); Z-Image: 4 (cos,sin) pairs of the element's
+// axis (metal/mqk_shader.zig:80-96).
+struct Rope8 { f32x4 a, b, c, d; };
+
+__device__ __forceinline__ Rope8 ld_rope8(const QkOps& a, int mode, const QkRow& r, int d0) {
+    Rope8 t;
+    if (mode == kQkKlein) {
+        t.a = *reinterpret_cast<const f32x4*>(r.cos_r + d0);
+        t.b = *reinterpret_cast<const f32x4*>(r.cos_r + d0 + 4);
+        t.c = *reinterpret_cast<const f32x4*>(r.sin_r + d0);
+        t.d = *reinterpret_cast<const f32x4*>(r.sin_r + d0 + 4);
+    } else {
+        const int d01 = a.dim0 + a.dim1;
+        const int axis = d0 < a.dim0 ? 0 : (d0 < d01 ? 1 : 2);
+        const int axis_off = axis == 0 ? 0 : (axis == 1 ? a.dim0 : d01);
+        const unsigned axis_pairs = (unsigned)(axis == 0 ? a.dim0 : (axis == 1 ? a.dim1 : a.dim2)) >> 1;
+        const unsigned base = axis == 0 ? a.base0 : (axis == 1 ? a.base1 : a.base2);
+        const unsigned long long p = axis == 0 ? r.p0 : (axis == 1 ? r.p1 : r.p2);
+        const unsigned long long idx = base + p * axis_pairs + (unsigned)((d0 - axis_off) >> 1);
+        const float* src = a.pairs + idx * 2;
+        t.a = *reinterpret_cast<const f32x4*>(src);      // (c0,s0,c1,s1)
+        t.b = *reinterpret_cast<const f32x4*>(src + 4);  // (c2,s2,c3,s3)
+        t.c = t.a;
+        t.d = t.b;
+    }
+    return t;
+}
+
+// x[0..7] (elements d0..d0+7 of a row) -> normalised, weighted, rotated.
+__device__ __forceinline__ void qk_apply8(int mode, float (&x)[8], float inv, const float* w, int d0, const Rope8& t) {
+    const f32x4 w0 = *reinterpret_cast<const f32x4*>(w + d0);
+    const f32x4 w1 = *reinterpret_cast<const f32x4*>(w + d0 + 4);
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        y[i] = x[i] * inv * w0[i];
+        y[4 + i] = x[4 + i] * inv * w1[i];
+    }
+    if (mode == kQkKlein) {
+        float c[8], s[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) { c[i] = t.a[i]; c[4 + i] = t.b[i]; s[i] = t.c[i]; s[4 + i] = t.d[i]; }
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+            x[i] = y[i] * c[i] - y[i + 1] * s[i];
+            x[i + 1] = y[i + 1] * c[i + 1] + y[i] * s[i + 1];
+        }
+    } else {
+        const float c[4] = {t.a[0], t.a[2], t.b[0], t.b[2]};
+        const float s[4] = {t.a[1], t.a[3], t.b[1], t.b[3]};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            x[2 * i] = y[2 * i] * c[i] - y[2 * i + 1] * s[i];
+            x[2 * i + 1] = y[2 * i + 1] * c[i] + y[2 * i] * s[i];
+        }
+    }
+}
+
+// Sum across the TPK adjacent lanes that share one K row (TPK = 4, 8 or 16).
+template <int TPK>
+__device__ __forceinline__ float row_group_sum(float v) {
+    // quad_perm [1,0,3,2], quad_perm [2,3,0,1], then row_half_mirror for 8, row_mirror for 16
+    v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0xB1, 0xF, 0xF, true));
+    v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x4E, 0xF, 0xF, true));
+    if constexpr (TPK >= 8)
+        v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x141, 0xF, 0xF, true));
+    if constexpr (TPK == 16) // row_mirror
+        v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x140, 0xF, 0xF, true));
+    return v;
+}
+
+} // namespace zdraw

@@ -94,4 +94,12 @@ hipError_t launch_qk_prepass(const PrepArgs& args, int in_dtype, hipStream_t str
 // One-time per-device setup (raises the dynamic LDS limit on every instantiation).
 hipError_t attention_setup();
 
+// The software-pipelined kernel (64 query rows per wave, 4 waves, 32-key blocks).
+// shape: 0 = two 32-query blocks per wave x 4 waves, 1 = one x 8 waves, 2 = one x 4 waves
+int attention_v2_block_rows(int shape);
+int attention_v2_key_block();
+int attention_v2_max_tokens();
+hipError_t launch_attention_v2(const AttnArgs& args, int in_dtype, int k_mode, int shape, hipStream_t stream);
+hipError_t attention_v2_setup();
+
 } // namespace zdraw

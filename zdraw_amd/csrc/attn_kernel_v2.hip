@@ -1,0 +1,585 @@
+// gfx950 flash-attention forward, software-pipelined form: 64 query rows per
+// wave, four waves per workgroup (256 query rows share every K/V block).
+//
+// Compared with the 32-rows-per-wave kernel this one
+//   * reuses each K fragment and each V fragment for two MFMAs (two 32-query
+//     blocks per wave), halving LDS reads per FLOP;
+//   * keeps V row-major in LDS and builds the V^T operand with the transposing
+//     LDS read (ds_read_b64_tr_b16), so staging V is a plain 16-byte copy;
+//   * walks the keys in blocks of 32 through a 4-stage LDS ring and overlaps,
+//     inside one wave, the MFMAs of S(b+1) = K(b+1) Q^T and O += V(b-1)^T P(b-1)
+//     with the softmax VALU work of block b (the three are independent), one
+//     barrier per block.
+// Block order is fixed; there are no atomics; results are bit-stable.
+#include "attn_device.hpp"
+
+namespace zdraw {
+
+namespace v2 {
+
+#ifndef ZDRAW_DIAG
+#define ZDRAW_DIAG 0 // timing experiments only: 1 no softmax VALU, 2 no MFMA, 4 no LDS fragment reads, 8 no barrier, 16 no staging
+#endif
+#ifndef ZDRAW_LDS_LOOKAHEAD
+#define ZDRAW_LDS_LOOKAHEAD 4
+#endif
+
+constexpr int KB = 32;            // keys per block
+constexpr int KPITCH = D + 8;     // 272 B rows: 16-lane b128 reads spread over all banks
+constexpr int VPITCH = D + 32;    // 320 B rows: a 32-lane transposing read covers 4 rows x 64 B without overlap
+constexpr int KS_ELEMS = KB * KPITCH;
+constexpr int VS_ELEMS = KB * VPITCH;
+constexpr int MAX_BLOCKS = 1024;  // key-block list capacity (tokens <= 32768)
+constexpr float kTau = 8.0f;             // log2 headroom of the lazy softmax maximum
+
+// Ring depth: 8 stages when one workgroup owns the CU (blocks are stored three
+// steps ahead of their first use, so one barrier per two steps orders every
+// write against its readers), 4 stages when two workgroups share the CU's LDS
+// (stored two steps ahead, one barrier per step).
+constexpr int ring_stages(int qb, int nw) { return (qb == 2 || nw == 8) ? 8 : 4; }
+constexpr size_t lds_bytes(int nst) {
+    return (size_t)nst * (KS_ELEMS + VS_ELEMS) * sizeof(bf16_t) + (size_t)MAX_BLOCKS * sizeof(unsigned short);
+}
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// Keeps a value's producer on this side of the point where it is called: the
+// empty volatile asm "uses and redefines" the register, so the optimiser can
+// neither sink the computation past it (into a later block) nor reorder it
+// with the scheduling fences, which are ordered with volatile asm.
+template <typename T>
+__device__ __forceinline__ void pin(T& v) {
+    asm volatile("" : "+v"(v));
+}
+
+// Four keys (rows) for this lane's head-dim column, from row-major V in LDS.
+// Within each 16-lane group the hardware returns to lane i, element j, the
+// value at (row of source lane (i>>2)+4j, column i&3 of that lane's 4-element
+// chunk); `p` must point at row (lane&15)>>2, chunk lane&3 of the 4x16 patch.
+__device__ __forceinline__ s16x4 lds_read_tr(const bf16_t* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(p)));
+}
+
+// QB = 32-query blocks per wave (1 or 2), NW = waves per workgroup.
+//   QB=2, NW=4: one wave per SIMD with the full 512-register budget;
+//   QB=1, NW=8: two waves per SIMD, 256 registers each;
+//   QB=1, NW=4: two workgroups per CU, each with its own LDS ring.
+template <typename TIn, int KMODE, bool MASKED, int QB, int NW>
+__global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel(const AttnArgs a) {
+    constexpr int NT = NW * 64;
+    constexpr int QR = 32 * QB;       // query rows per wave
+    constexpr int BQ = NW * QR;       // query rows per workgroup
+    constexpr int CPT = 512 / NT;     // 8-element chunks of K (and of V) per thread per block
+    constexpr int TPK = 16 / CPT;     // threads sharing one key row
+    constexpr int NST = ring_stages(QB, NW);
+    constexpr int AHEAD = NST == 8 ? 3 : 2;   // a block is stored AHEAD steps before S needs its K
+    constexpr int LA = ZDRAW_LDS_LOOKAHEAD;   // slots between an LDS fragment read and its MFMA
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    bf16_t* const Ks = reinterpret_cast<bf16_t*>(smem);
+    bf16_t* const Vs = Ks + NST * KS_ELEMS;
+    unsigned short* const blocks = reinterpret_cast<unsigned short*>(Vs + NST * VS_ELEMS);
+    __shared__ int s_nblocks;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+
+    // XCD-aware remap: consecutive logical ids (one head's query blocks) share an XCD's L2
+    int logical;
+    {
+        const int nwg = gridDim.x;
+        const int xcd = blockIdx.x & 7;
+        const int idx = blockIdx.x >> 3;
+        const int base = nwg >> 3;
+        const int rem = nwg & 7;
+        logical = idx + xcd * base + (xcd < rem ? xcd : rem);
+    }
+    const int bh = logical / a.nqb;
+    const int qb = logical - bh * a.nqb;
+    const int seg = bh / a.heads;
+    const int head = bh - seg * a.heads;
+    const int q0 = qb * BQ + wave * QR;
+
+    // zero the ring: the pipeline's first O update and last S update touch
+    // stages that no block has been stored to yet
+    {
+        u32x4* z = reinterpret_cast<u32x4*>(smem);
+        const int n16 = (int)((size_t)NST * (KS_ELEMS + VS_ELEMS) * sizeof(bf16_t) / 16);
+        for (int i = tid; i < n16; i += NT) z[i] = u32x4{0u, 0u, 0u, 0u};
+    }
+
+    // ---- key-block list: blocks with at least one admitted key, ascending
+    const int nb_all = (a.key_limit + KB - 1) / KB;
+    const unsigned char* const kp = a.key_pad ? a.key_pad + (int64_t)seg * a.mask_bs : nullptr;
+    int nblk = nb_all;
+    if (MASKED && kp) {
+        if (wave == 0) {
+            int count = 0;
+            for (int base = 0; base < nb_all; base += 64) {
+                const int t = base + lane;
+                bool act = false;
+                if (t < nb_all) {
+                    const int k0 = t * KB;
+                    const int k1 = min(k0 + KB, a.key_limit);
+                    for (int j = k0; j < k1; j++) act |= (kp[j] == 0);
+                }
+                const unsigned long long m = __ballot(act);
+                if (act) blocks[count + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short)t;
+                count += __popcll(m);
+            }
+            if (lane == 0) s_nblocks = count;
+        }
+        __syncthreads();
+        nblk = s_nblocks;
+    }
+    auto block_of = [&](int i) -> int { return (MASKED && kp) ? (int)blocks[i] : i; };
+
+    // ---- Q rows -> B-operand registers: qf[qi][s], lane: query 32*qi + l32, dims 16s + 8h .. +7
+    bf16x8 qf[QB][8];
+#pragma unroll
+    for (int qi = 0; qi < QB; qi++) {
+        const int qrow = q0 + 32 * qi + l32;
+        const bool ok = qrow < a.tokens;
+        const TIn* qp = reinterpret_cast<const TIn*>(a.q) + (int64_t)seg * a.q_bs + (int64_t)(ok ? qrow : 0) * a.q_ts +
+                        (int64_t)head * a.q_hs + 8 * h;
+        float x[8][8];
+#pragma unroll
+        for (int s = 0; s < 8; s++) unpack8(ld_raw8<TIn>(qp + 16 * s, ok), x[s]);
+        if (a.q_mode != kQkNone) {
+            float ss = 0.f;
+#pragma unroll
+            for (int s = 0; s < 8; s++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) ss += x[s][i] * x[s][i];
+            ss = pair_sum(ss);
+            const float inv = rsqrtf(ss * (1.0f / D) + a.qk.eps);
+            const QkRow r = qk_row(a.qk, a.q_mode, a.q_w, a.q_w_txt, seg, qrow, ok);
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const int d0 = 16 * s + 8 * h;
+                const Rope8 t = ld_rope8(a.qk, a.q_mode, r, d0);
+                qk_apply8(a.q_mode, x[s], inv, r.w, d0, t);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 8; s++) qf[qi][s] = __builtin_bit_cast(bf16x8, pack_bf16x8(x[s]));
+    }
+
+    // ---- block staging: thread t owns key t/TPK of the block, CPT chunks of 8 dims of K and of V
+    const int lk_key = tid / TPK;
+    const int lk_d0 = (tid % TPK) * CPT * 8;
+    const TIn* const kbase = reinterpret_cast<const TIn*>(a.k) + (int64_t)seg * a.k_bs + (int64_t)head * a.k_hs + lk_d0;
+    const TIn* const vbase = reinterpret_cast<const TIn*>(a.v) + (int64_t)seg * a.v_bs + (int64_t)head * a.v_hs + lk_d0;
+
+    Raw8<TIn> kraw[CPT], vraw[CPT];
+    Rope8 krope[KMODE == kQkNone ? 1 : CPT];
+    QkRow krow;
+
+    // i = position in the block list. Loads are unconditional (no branches in
+    // the pipelined loop): positions past the end re-read the last block and
+    // rows past the sequence re-read its last row. Neither is ever used: the
+    // drained ring stages feed only discarded MFMAs, and keys past the limit
+    // are masked to -inf before the softmax.
+    const int last_row = a.tokens - 1;
+    auto stage_load = [&](int i) {
+        const int ii = i < nblk ? i : nblk - 1;
+        int key = block_of(ii) * KB + lk_key;
+        key = key < last_row ? key : last_row;
+        const TIn* pk = kbase + (int64_t)key * a.k_ts;
+        const TIn* pv = vbase + (int64_t)key * a.v_ts;
+#pragma unroll
+        for (int c = 0; c < CPT; c++) {
+            kraw[c] = ld_raw8<TIn>(pk + 8 * c, true);
+            vraw[c] = ld_raw8<TIn>(pv + 8 * c, true);
+        }
+        if constexpr (KMODE != kQkNone) {
+            krow = qk_row(a.qk, KMODE, a.k_w, a.k_w_txt, seg, key, true);
+#pragma unroll
+            for (int c = 0; c < CPT; c++) krope[c] = ld_rope8(a.qk, KMODE, krow, lk_d0 + 8 * c);
+        }
+    };
+
+    auto stage_store = [&](int stage) {
+        bf16_t* kdst = Ks + stage * KS_ELEMS + lk_key * KPITCH + lk_d0;
+        bf16_t* vdst = Vs + stage * VS_ELEMS + lk_key * VPITCH + lk_d0;
+        if constexpr (KMODE == kQkNone) {
+#pragma unroll
+            for (int c = 0; c < CPT; c++) *reinterpret_cast<u32x4*>(kdst + 8 * c) = raw_to_bf16(kraw[c]);
+        } else {
+            float x[CPT][8];
+            float ss = 0.f;
+#pragma unroll
+            for (int c = 0; c < CPT; c++) {
+                unpack8(kraw[c], x[c]);
+#pragma unroll
+                for (int i = 0; i < 8; i++) ss += x[c][i] * x[c][i];
+            }
+            ss = row_group_sum<TPK>(ss);
+            const float inv = rsqrtf(ss * (1.0f / D) + a.qk.eps);
+#pragma unroll
+            for (int c = 0; c < CPT; c++) {
+                qk_apply8(KMODE, x[c], inv, krow.w, lk_d0 + 8 * c, krope[c]);
+                *reinterpret_cast<u32x4*>(kdst + 8 * c) = pack_bf16x8(x[c]);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CPT; c++) *reinterpret_cast<u32x4*>(vdst + 8 * c) = raw_to_bf16(vraw[c]);
+    };
+
+    // ---- running state
+    f32x16 oacc[QB][4]; // O^T: lane query 32*qi + l32, dims 32*blk + 8i + 4h + j
+#pragma unroll
+    for (int qi = 0; qi < QB; qi++)
+#pragma unroll
+        for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+            for (int j = 0; j < 16; j++) oacc[qi][blk][j] = 0.f;
+    float m_run[QB], l_run[QB]; // running maximum (already multiplied by scale_log2) and denominator half
+#pragma unroll
+    for (int qi = 0; qi < QB; qi++) {
+        m_run[qi] = -INFINITY;
+        l_run[qi] = 0.f;
+    }
+
+    // S^T block = K(block) . Q^T for both query blocks
+    auto qk_block = [&](int stage, f32x16 (&s_out)[QB]) {
+#pragma unroll
+        for (int qi = 0; qi < QB; qi++)
+#pragma unroll
+            for (int j = 0; j < 16; j++) s_out[qi][j] = 0.f;
+        const bf16_t* kt = Ks + stage * KS_ELEMS + l32 * KPITCH + 8 * h;
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kt + 16 * s);
+#pragma unroll
+            for (int qi = 0; qi < QB; qi++)
+                s_out[qi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qi][s], s_out[qi], 0, 0, 0);
+        }
+    };
+
+    // O^T += V(block)^T . P^T
+    const int tr_row = (lane & 15) >> 2;
+    const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    auto pv_block = [&](int stage, const bf16x8 (&p)[QB][2]) {
+        const bf16_t* vt = Vs + stage * VS_ELEMS + (4 * h + tr_row) * VPITCH + tr_col;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int blk = 0; blk < 4; blk++) {
+                const s16x4 lo = lds_read_tr(vt + (16 * kb) * VPITCH + 32 * blk);
+                const s16x4 hi = lds_read_tr(vt + (16 * kb + 8) * VPITCH + 32 * blk);
+                typedef short s16x8 __attribute__((ext_vector_type(8)));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
+#pragma unroll
+                for (int qi = 0; qi < QB; qi++)
+                    oacc[qi][blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p[qi][kb], oacc[qi][blk], 0, 0, 0);
+            }
+        }
+    };
+
+    // One pipeline step for list position b: consumes S(b) and P(b-1),
+    // produces S(b+1) and P(b). The three streams are independent, so the
+    // step is laid out by hand as 16 slots, each fenced from the next:
+    //   LDS reads for the MFMA two slots ahead | one MFMA per query block |
+    //   one slice of the softmax VALU work, which runs in the MFMA's shadow.
+    // Even slots extend S(b+1) = K(b+1) Q^T, odd slots add V(b-1)^T P(b-1)^T to O^T.
+    auto step = [&](int b, bool sync, f32x16 (&s_cur)[QB], f32x16 (&s_next)[QB], const bf16x8 (&p_prev)[QB][2],
+                    bf16x8 (&p_cur)[QB][2]) __attribute__((always_inline)) {
+        // ring: block b+AHEAD (in registers since the previous step) goes to its stage,
+        // whose previous tenant's last reader (V, NST-AHEAD-1 steps back) is at least one
+        // barrier behind; then the loads of block b+AHEAD+1 start
+        if (!(ZDRAW_DIAG & 16)) {
+            stage_store((b + AHEAD) & (NST - 1));
+            stage_load(b + AHEAD + 1);
+        }
+
+        const bf16_t* kt = Ks + ((b + 1) & (NST - 1)) * KS_ELEMS + l32 * KPITCH + 8 * h;
+        const bf16_t* vt = Vs + ((b + NST - 1) & (NST - 1)) * VS_ELEMS + (4 * h + tr_row) * VPITCH + tr_col;
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        bf16x8 kf[8];
+        s16x4 vlo[8], vhi[8];
+        if (ZDRAW_DIAG & 4) {
+            for (int i = 0; i < 8; i++) { kf[i] = qf[0][i]; vlo[i] = s16x4{1, 2, 3, 4}; vhi[i] = vlo[i]; }
+        }
+        auto read_slot = [&](int slot) __attribute__((always_inline)) {
+            if (ZDRAW_DIAG & 4) return;
+            if (slot & 1) {
+                const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
+                vlo[idx] = lds_read_tr(vt + (16 * kb) * VPITCH + 32 * blk);
+                vhi[idx] = lds_read_tr(vt + (16 * kb + 8) * VPITCH + 32 * blk);
+            } else {
+                kf[slot >> 1] = *reinterpret_cast<const bf16x8*>(kt + 16 * (slot >> 1));
+            }
+        };
+        auto mfma_slot = [&](int slot) __attribute__((always_inline)) {
+            if (ZDRAW_DIAG & 2) return;
+            if (slot & 1) {
+                const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
+                const bf16x8 vf =
+                    __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(vlo[idx], vhi[idx], 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+                for (int qi = 0; qi < QB; qi++)
+                    oacc[qi][blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_prev[qi][kb], oacc[qi][blk], 0, 0, 0);
+            } else {
+                const int st = slot >> 1;
+#pragma unroll
+                for (int qi = 0; qi < QB; qi++)
+                    s_next[qi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[qi][st], s_next[qi], 0, 0, 0);
+            }
+        };
+
+        if constexpr (MASKED) {
+            // excluded keys (padding mask, key limit, tail) -> -inf; bit kk of badm = key kk of the block
+            const int key = block_of(b) * KB + l32;
+            const bool bad = key >= a.key_limit || (kp != nullptr && kp[key < a.key_limit ? key : 0] != 0);
+            const unsigned badm = (unsigned)__ballot(bad); // lanes 0..31 carry the block's 32 keys
+#pragma unroll
+            for (int qi = 0; qi < QB; qi++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int kk = 8 * i + 4 * h + j;
+                        s_cur[qi][4 * i + j] = ((badm >> kk) & 1u) ? -INFINITY : s_cur[qi][4 * i + j];
+                    }
+        }
+#pragma unroll
+        for (int qi = 0; qi < QB; qi++)
+#pragma unroll
+            for (int j = 0; j < 16; j++) s_next[qi][j] = 0.f;
+
+        float t[QB][7], mc[QB], alpha[QB], psum[QB];
+        unsigned pc[QB][8] = {}; // P as packed bf16 pairs
+        bool grew = false;
+        if (ZDRAW_DIAG & 1) {
+            for (int qi = 0; qi < QB; qi++) { alpha[qi] = 1.f; p_cur[qi][0] = p_prev[qi][0]; p_cur[qi][1] = p_prev[qi][1]; }
+        }
+        // softmax of S(b) in 16 slices (per query block)
+        auto valu_slice = [&](int c) __attribute__((always_inline)) {
+            if (ZDRAW_DIAG & 1) return;
+            if ((ZDRAW_DIAG & 32) && c >= 7 && c <= 10) return; // half of the exponentials
+#pragma unroll
+            for (int qi = 0; qi < QB; qi++) {
+                f32x16& sv = s_cur[qi];
+                if (c == 0) {
+                    t[qi][0] = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
+                    t[qi][1] = fmaxf(fmaxf(sv[3], sv[4]), sv[5]);
+                    t[qi][2] = fmaxf(fmaxf(sv[6], sv[7]), sv[8]);
+                    t[qi][3] = fmaxf(fmaxf(sv[9], sv[10]), sv[11]);
+                } else if (c == 1) {
+                    t[qi][4] = fmaxf(fmaxf(sv[12], sv[13]), sv[14]);
+                    t[qi][5] = fmaxf(fmaxf(t[qi][0], t[qi][1]), t[qi][2]);
+                    t[qi][6] = fmaxf(fmaxf(t[qi][3], t[qi][4]), sv[15]);
+                    t[qi][0] = fmaxf(t[qi][5], t[qi][6]);
+                } else if (c == 2) {
+                    // Lazy running maximum, kept in the exp2 domain: the reference point of
+                    // the exponentials only moves when this block's maximum exceeds it by
+                    // more than kTau, so P stays within [0, 2^kTau] and O is rescaled on a
+                    // handful of blocks instead of on every new row maximum.
+                    const float mlc = pair_max(t[qi][0]) * a.scale_log2;
+                    const bool up = mlc > m_run[qi] + kTau;
+                    const float m_new = up ? mlc : m_run[qi];
+                    mc[qi] = (m_new == -INFINITY) ? 0.f : m_new;
+                    alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - mc[qi]);
+                    grew |= up;
+                    m_run[qi] = m_new;
+                    psum[qi] = 0.f;
+                    pin(mc[qi]);
+                    pin(alpha[qi]);
+                } else if (c <= 10) {
+                    const int e = 2 * (c - 3); // elements e, e+1 of 16
+                    f32x2 pp;
+                    pp[0] = __builtin_amdgcn_exp2f(sv[e] * a.scale_log2 - mc[qi]);
+                    pp[1] = __builtin_amdgcn_exp2f(sv[e + 1] * a.scale_log2 - mc[qi]);
+                    const bf16x2 pr = __builtin_convertvector(pp, bf16x2);
+                    // the denominator sums the same bf16-rounded weights the MFMA multiplies by
+                    psum[qi] = __builtin_amdgcn_fdot2_f32_bf16(pr, bf16x2{(bf16_t)1.0f, (bf16_t)1.0f}, psum[qi], false);
+                    pc[qi][e >> 1] = __builtin_bit_cast(unsigned, pr);
+                    pin(psum[qi]);
+                    pin(pc[qi][e >> 1]);
+                } else if (c == 12) {
+                    p_cur[qi][0] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][0], pc[qi][1], pc[qi][2], pc[qi][3]});
+                    p_cur[qi][1] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][4], pc[qi][5], pc[qi][6], pc[qi][7]});
+                } else if (c == 14) {
+                    l_run[qi] = l_run[qi] * alpha[qi] + psum[qi];
+                    pin(l_run[qi]);
+                }
+            }
+        };
+
+        // LDS reads run LA slots ahead of the MFMA that consumes them
+#pragma unroll
+        for (int g = 0; g < LA; g++) read_slot(g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < 16; g++) {
+            if (g + LA < 16) read_slot(g + LA);
+            mfma_slot(g);
+            valu_slice(g);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // O is relative to m(b-1) here; move it to m(b) before block b's update lands
+        if (__any(grew)) {
+#pragma unroll
+            for (int qi = 0; qi < QB; qi++)
+#pragma unroll
+                for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                    for (int j = 0; j < 16; j++) oacc[qi][blk][j] *= alpha[qi];
+        }
+        if (sync && !(ZDRAW_DIAG & 8)) __syncthreads();
+    };
+
+    if (nblk > 0) {
+        // prologue: blocks 0 .. AHEAD-1 into the ring, block AHEAD in flight
+        stage_load(0);
+        __syncthreads(); // ring zeroing complete
+#pragma unroll
+        for (int i = 0; i < AHEAD; i++) {
+            stage_store(i);
+            stage_load(i + 1);
+        }
+        __syncthreads();
+
+        f32x16 s_a[QB], s_b[QB];
+        bf16x8 p_a[QB][2], p_b[QB][2];
+#pragma unroll
+        for (int qi = 0; qi < QB; qi++)
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) p_a[qi][kb][j] = (bf16_t)0.0f;
+        qk_block(0, s_a);
+
+        // two steps per trip so the S and P buffers swap roles without copies; with the
+        // 8-stage ring only the second step of a trip ends in a barrier
+        int b = 0;
+        for (; b + 1 < nblk; b += 2) {
+            step(b, NST != 8, s_a, s_b, p_a, p_b);
+            step(b + 1, true, s_b, s_a, p_b, p_a);
+        }
+        if (b < nblk) {
+            step(b, true, s_a, s_b, p_a, p_b);
+            pv_block((nblk - 1) & (NST - 1), p_b);
+        } else {
+            pv_block((nblk - 1) & (NST - 1), p_a);
+        }
+    }
+
+    // ---- epilogue: O = O^T / l
+#pragma unroll
+    for (int qi = 0; qi < QB; qi++) {
+        const float l_tot = pair_sum(l_run[qi]);
+        const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        const int qrow = q0 + 32 * qi + l32;
+        if (qrow < a.tokens) {
+            const int64_t off = (int64_t)seg * a.o_bs + (int64_t)qrow * a.o_ts + (int64_t)head * a.o_hs;
+            if (a.out_dtype == kF32) {
+                float* op = reinterpret_cast<float*>(a.o) + off;
+#pragma unroll
+                for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        f32x4 v;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
+                        *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
+                    }
+            } else {
+                bf16_t* op = reinterpret_cast<bf16_t*>(a.o) + off;
+#pragma unroll
+                for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        f32x4 v;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
+                        *reinterpret_cast<bf16x4*>(op + 32 * blk + 8 * i + 4 * h) = __builtin_convertvector(v, bf16x4);
+                    }
+            }
+        }
+    }
+}
+
+template <typename TIn, int KMODE, bool MASKED, int QB, int NW>
+static hipError_t launch_one(const AttnArgs& a, hipStream_t stream) {
+    const int64_t nwg = (int64_t)a.nqb * a.heads * a.batch;
+    if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
+    attn_fwd_v2_kernel<TIn, KMODE, MASKED, QB, NW>
+        <<<dim3((unsigned)nwg), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
+    return hipGetLastError();
+}
+
+template <typename TIn, bool MASKED, int QB, int NW>
+static hipError_t launch_kmode(const AttnArgs& a, int k_mode, hipStream_t stream) {
+    switch (k_mode) {
+    case kQkNone: return launch_one<TIn, kQkNone, MASKED, QB, NW>(a, stream);
+    case kQkKlein: return launch_one<TIn, kQkKlein, MASKED, QB, NW>(a, stream);
+    case kQkZimage: return launch_one<TIn, kQkZimage, MASKED, QB, NW>(a, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <int QB, int NW>
+static hipError_t launch_shape(const AttnArgs& a, int in_dtype, int k_mode, hipStream_t stream) {
+    // the masked build is only needed when some key of some block is excluded
+    const bool masked = a.key_pad != nullptr || (a.key_limit % KB) != 0;
+    if (in_dtype == kF32)
+        return masked ? launch_kmode<float, true, QB, NW>(a, k_mode, stream)
+                      : launch_kmode<float, false, QB, NW>(a, k_mode, stream);
+    if (in_dtype == kBF16)
+        return masked ? launch_kmode<bf16_t, true, QB, NW>(a, k_mode, stream)
+                      : launch_kmode<bf16_t, false, QB, NW>(a, k_mode, stream);
+    return hipErrorInvalidValue;
+}
+
+template <typename TIn, int KMODE, bool MASKED, int QB, int NW>
+static hipError_t raise_lds() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_v2_kernel<TIn, KMODE, MASKED, QB, NW>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(ring_stages(QB, NW)));
+}
+
+template <int QB, int NW>
+static hipError_t raise_shape() {
+    hipError_t e;
+#define ZD_RAISE(T, M) \
+    if ((e = raise_lds<T, M, false, QB, NW>()) != hipSuccess) return e; \
+    if ((e = raise_lds<T, M, true, QB, NW>()) != hipSuccess) return e;
+    ZD_RAISE(float, kQkNone) ZD_RAISE(float, kQkKlein) ZD_RAISE(float, kQkZimage)
+    ZD_RAISE(bf16_t, kQkNone) ZD_RAISE(bf16_t, kQkKlein) ZD_RAISE(bf16_t, kQkZimage)
+#undef ZD_RAISE
+    return hipSuccess;
+}
+
+} // namespace v2
+
+// shape: 0 = 2 query blocks x 4 waves, 1 = 1 x 8, 2 = 1 x 4
+int attention_v2_block_rows(int shape) { return shape == 0 ? 256 : (shape == 1 ? 256 : 128); }
+int attention_v2_key_block() { return v2::KB; }
+int attention_v2_max_tokens() { return v2::MAX_BLOCKS * v2::KB; }
+
+hipError_t launch_attention_v2(const AttnArgs& a, int in_dtype, int k_mode, int shape, hipStream_t stream) {
+    switch (shape) {
+    case 0: return v2::launch_shape<2, 4>(a, in_dtype, k_mode, stream);
+    case 1: return v2::launch_shape<1, 8>(a, in_dtype, k_mode, stream);
+    case 2: return v2::launch_shape<1, 4>(a, in_dtype, k_mode, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t attention_v2_setup() {
+    hipError_t e;
+    if ((e = v2::raise_shape<2, 4>()) != hipSuccess) return e;
+    if ((e = v2::raise_shape<1, 8>()) != hipSuccess) return e;
+    if ((e = v2::raise_shape<1, 4>()) != hipSuccess) return e;
+    return hipSuccess;
+}
+
+} // namespace zdraw

@@ -55,7 +55,7 @@ uint64_t g_dispatch = 0;
 uint64_t g_command = 0;
 uint64_t g_fallback = 0;
 uint64_t g_gpu_ns = 0;
-int g_waves = 8;
+int g_variant = 0; // 0..2: pipelined kernel shapes (2x4, 1x8, 1x4 query blocks x waves); 3, 4: unpipelined kernel, 8 / 4 waves
 bool g_setup_done = false;
 
 thread_local char g_err[512] = "";
@@ -154,7 +154,8 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     if (p->causal != 0) return unavailable("causal attention");
     if (p->kv_heads != p->heads) return unavailable("grouped-query attention");
     if (x->batch == 0) return invalid("batch == 0");
-    if ((uint64_t)p->tokens > (uint64_t)kMaxKeyTiles * kKeyTile) return unavailable("too many tokens");
+    const uint64_t max_tokens = g_variant <= 2 ? (uint64_t)attention_v2_max_tokens() : (uint64_t)kMaxKeyTiles * kKeyTile;
+    if ((uint64_t)p->tokens > max_tokens) return unavailable("too many tokens");
     if ((x->in_dtype != ZDRAW_HIP_F32 && x->in_dtype != ZDRAW_HIP_BF16) ||
         (x->out_dtype != ZDRAW_HIP_F32 && x->out_dtype != ZDRAW_HIP_BF16))
         return unavailable("activation dtype");
@@ -184,7 +185,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     a.heads = (int32_t)p->heads;
     a.batch = (int32_t)x->batch;
     a.key_limit = (int32_t)((p->valid != 0 && p->valid < p->tokens) ? p->valid : p->tokens);
-    const int rows = attention_block_rows(g_waves);
+    const int rows = g_variant <= 2 ? attention_v2_block_rows(g_variant) : attention_block_rows(g_variant == 3 ? 8 : 4);
     a.nqb = (int32_t)((p->tokens + rows - 1) / rows);
     a.q_mode = (int32_t)x->qk_mode;
     a.out_dtype = (int32_t)x->out_dtype;
@@ -283,6 +284,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
 int enqueue(const FusedPlan& plan, hipStream_t stream) {
     if (!g_setup_done) {
         hipError_t e = attention_setup();
+        if (e == hipSuccess) e = attention_v2_setup();
         if (e != hipSuccess) {
             set_err("attention_setup: %s", hipGetErrorString(e));
             return ZDRAW_HIP_ERR_HANDLE;
@@ -297,7 +299,8 @@ int enqueue(const FusedPlan& plan, hipStream_t stream) {
         }
         g_dispatch++;
     }
-    hipError_t e = launch_attention(plan.args, plan.in_dtype, plan.k_mode, g_waves, stream);
+    hipError_t e = g_variant <= 2 ? launch_attention_v2(plan.args, plan.in_dtype, plan.k_mode, g_variant, stream)
+                                  : launch_attention(plan.args, plan.in_dtype, plan.k_mode, g_variant == 3 ? 8 : 4, stream);
     if (e != hipSuccess) {
         set_err("attention launch: %s", hipGetErrorString(e));
         return ZDRAW_HIP_ERR_HANDLE;
@@ -383,6 +386,8 @@ void* zdraw_hip_create_device(void) {
         return nullptr;
     }
     if (hipSetDevice(0) != hipSuccess) return nullptr;
+    // ZDRAW_ATTN_VARIANT picks the kernel build for a whole process (measurement aid)
+    if (const char* v = getenv("ZDRAW_ATTN_VARIANT")) zdraw_hip_set_attention_variant(atoi(v));
     Device* d = new Device{0};
     return d;
 }
@@ -480,7 +485,7 @@ void zdraw_hip_release_pipeline(void* pipeline) { delete static_cast<Pipeline*>(
 size_t zdraw_hip_pipeline_threads(void* pipeline) {
     Pipeline* p = static_cast<Pipeline*>(pipeline);
     if (!p) return 0;
-    return p->kind == 0 ? (size_t)g_waves * 64 : 256;
+    return p->kind == 0 ? ((g_variant == 1 || g_variant == 3) ? 512 : 256) : 256;
 }
 
 // ---------------------------------------------------------------- attention
@@ -712,7 +717,7 @@ int zdraw_hip_queue_sync(void* queue) {
     return e == hipSuccess ? ZDRAW_HIP_OK : hip_fail(e, "queue sync");
 }
 
-void zdraw_hip_set_attention_waves(int nwaves) { g_waves = (nwaves == 4) ? 4 : 8; }
+void zdraw_hip_set_attention_variant(int variant) { g_variant = (variant >= 0 && variant <= 4) ? variant : 0; }
 
 size_t zdraw_hip_abi_sizeof(int which) {
     switch (which) {

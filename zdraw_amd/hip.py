@@ -5,7 +5,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libzdraw_hip.so")
+# ZDRAW_HIP_LIB points the binding at an experimental build of the same C ABI
+LIB_PATH = os.environ.get("ZDRAW_HIP_LIB") or os.path.join(HERE, "lib", "libzdraw_hip.so")
 
 OK, ERR_HANDLE, ERR_DEVICE, UNAVAILABLE, INVALID = 0, -1, -2, 1, 2
 K_ROWS, K_FLASH, K_BLOCK, K_WIDE = 0, 1, 2, 3
@@ -78,7 +79,7 @@ SYMBOLS = {
     "zdraw_hip_event_elapsed_ms": (C.c_float, [_vp, _vp]),
     "zdraw_hip_event_release": (None, [_vp]),
     "zdraw_hip_queue_sync": (_int, [_vp]),
-    "zdraw_hip_set_attention_waves": (None, [_int]),
+    "zdraw_hip_set_attention_variant": (None, [_int]),
     "zdraw_hip_abi_sizeof": (_sz, [_int]),
     "zdraw_hip_last_error": (C.c_char_p, []),
 }
