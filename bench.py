@@ -57,15 +57,45 @@ def cpu_baseline(w, seconds_target=15.0):
     }
 
 
+def timed_region(L, ctx, res, steps):
+    """K launches back to back on the library's stream, bracketed by a full
+    synchronisation on both sides (wall clock); the attention kernel of every
+    launch is bracketed by its own HIP events on that stream (device time)."""
+    L.zdraw_hip_queue_sync(ctx.queue)
+    L.zdraw_hip_metrics_reset()
+    L.zdraw_hip_trace_attention(1)
+    t0 = time.perf_counter()
+    b = L.zdraw_hip_batch_begin(ctx.queue)
+    for _ in range(steps):
+        rc = res.launch(b)
+        if rc != 0:
+            raise RuntimeError(f"launch rc={rc}")
+    if L.zdraw_hip_batch_end(b) != 0:
+        raise RuntimeError("batch_end failed")
+    L.zdraw_hip_queue_sync(ctx.queue)
+    wall = time.perf_counter() - t0
+    n = C.c_uint64(0)
+    kern_ns = L.zdraw_hip_trace_attention_ns(C.byref(n))
+    L.zdraw_hip_trace_attention(0)
+    if n.value != steps:
+        raise RuntimeError(f"traced {n.value} attention launches, expected {steps}")
+    return wall, kern_ns / 1e6 / steps
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="klein_1024")
-    ap.add_argument("--k-site", choices=["tile", "prepass"], default=os.environ.get("ZDRAW_BENCH_K_SITE", "tile"))
-    ap.add_argument("--variant", type=int, default=0, help="kernel build: 0 default, 1/2 the 32-row kernel")
+    ap.add_argument("--k-site", choices=["tile", "prepass"], default=os.environ.get("ZDRAW_BENCH_K_SITE", "prepass"),
+                    help="where K's norm+rope runs: inside the K-block load, or one pre-pass kernel per call")
+    ap.add_argument("--variant", type=int, default=0, help="kernel shape: 0 = 8 waves, 1 = 4 waves x 2 workgroups")
+    ap.add_argument("--dynamic-max", action="store_true", help="withhold the score bound (running-maximum softmax)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (a known-size kernel to scale "
+                         "the profiler's FETCH_SIZE / WRITE_SIZE counters against)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)")
@@ -79,49 +109,32 @@ def main():
     L.zdraw_hip_set_attention_variant(args.variant)
     w = wl.by_name(args.workload, seed=0)
     k_site = hip.K_PREPASS if args.k_site == "prepass" else hip.K_IN_TILE_LOAD
-    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=k_site)
-
-    def enqueue(n):
-        b = L.zdraw_hip_batch_begin(ctx.queue)
-        for _ in range(n):
-            rc = res.launch(b)
-            if rc != 0:
-                raise RuntimeError(f"launch rc={rc}: {hip.last_error()}")
-        return b
+    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=k_site, bounded=not args.dynamic_max)
 
     # warm-up (untimed)
-    if L.zdraw_hip_batch_end(enqueue(args.warmup)) != 0:
-        raise RuntimeError(hip.last_error())
-    L.zdraw_hip_queue_sync(ctx.queue)
-
-    # timed region: K launches back to back on the library's stream, bracketed
-    # by a full synchronisation on both sides (wall clock) and by HIP events
-    # recorded on that same stream (device time of the launches).
-    ev0, ev1 = L.zdraw_hip_event_create(), L.zdraw_hip_event_create()
-    L.zdraw_hip_queue_sync(ctx.queue)
-    t0 = time.perf_counter()
-    L.zdraw_hip_event_record(ev0, ctx.queue)
-    b = enqueue(args.steps)
-    L.zdraw_hip_event_record(ev1, ctx.queue)
-    if L.zdraw_hip_batch_end(b) != 0:
-        raise RuntimeError(hip.last_error())
-    L.zdraw_hip_queue_sync(ctx.queue)
-    wall = time.perf_counter() - t0
-    dev_ms = L.zdraw_hip_event_elapsed_ms(ev0, ev1)
-    L.zdraw_hip_event_release(ev0)
-    L.zdraw_hip_event_release(ev1)
+    timed_region(L, ctx, res, max(args.warmup, 1))
+    wall, kern_ms = timed_region(L, ctx, res, args.steps)
 
     out = res.read_output()
     if not np.isfinite(out).all():
         raise RuntimeError("non-finite output")
+
+    # the other K site, for the record (short, untimed by the driver's clock)
+    other = "tile" if args.k_site == "prepass" else "prepass"
+    res.ext.k_site = hip.K_IN_TILE_LOAD if other == "tile" else hip.K_PREPASS
+    timed_region(L, ctx, res, 3)
+    o_wall, _ = timed_region(L, ctx, res, 10)
 
     desc = (f"{w.name}: B={w.batch} H={w.heads} S={w.tokens} D=128 bf16, fused QK-RMSNorm + axial RoPE, "
             + ("no mask" if w.key_pad is None else "ragged key-padding mask"))
     flops = w.flops
     ms_per_step = wall * 1e3 / args.steps
     value = flops / (wall / args.steps) / 1e12
-    kern_ms = dev_ms / args.steps
     achieved = flops / (kern_ms * 1e-3) / 1e12
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", f"attn_fwd_{w.name}_traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
     line = {
         "metric": "attn TFLOP/s + % of bf16 MFMA peak, Klein 1024^2 (H=24,S=4608,D=128)",
         "value": value,
@@ -138,8 +151,10 @@ def main():
         "config": {
             "workload": desc,
             "k_norm_rope_site": args.k_site,
+            "softmax": "running maximum" if args.dynamic_max else "bounded scores (QK-norm bound supplied by the caller)",
             "kernel_variant": args.variant,
             "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
+            f"tflops_with_k_site_{other}": flops / (o_wall / 10) / 1e12,
         },
         "roofline": {
             "bound": "mfma",
@@ -147,13 +162,23 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_BF16_TFLOPS,
-            "traffic": None,
-            "kernel": "attn_fwd_kernel" + (" (+ qk_prepass_kernel in the same events)" if args.k_site == "prepass" else ""),
+            "traffic": traffic,
+            "kernel": "attn_fwd_kernel",
             "kernel_ms": kern_ms,
         },
     }
     res.release()
     ctx.deinit()
+    if args.copy_calibration_mib:
+        import torch
+
+        n = args.copy_calibration_mib << 20
+        src = torch.full((n,), 3, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads n bytes, writes n bytes
+        torch.cuda.synchronize()
+        line["config"]["copy_calibration_bytes"] = n
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(line), flush=True)

@@ -94,6 +94,14 @@ typedef struct ZdrawHipAttnExt {
     uint32_t k_site;           /* ZDRAW_HIP_K_IN_TILE_LOAD or ZDRAW_HIP_K_PREPASS */
     uint32_t txt_rows;         /* tokens < txt_rows use the *_txt weights (Klein double block) */
     float eps;                 /* RMSNorm epsilon */
+    /* Caller's upper bound on |q'.k'|/sqrt(head_dim) over all rows AFTER norm and
+     * rope, or 0 if unknown. With RMS-normalised Q and K and rope tables that are
+     * rotations it is sqrt(head_dim) * max|w_q| * max|w_k|. A bound of at most 44
+     * lets the kernel exponentiate scores without tracking a running maximum
+     * (softmax is shift-invariant); 0 or a larger bound selects the running-maximum
+     * form. A bound that is too small is a caller error (overflow). */
+    float score_bound;
+    uint32_t reserved;
 } ZdrawHipAttnExt;
 
 /* Buffer handles for the fused entry's side operands (NULL where unused). */
@@ -186,6 +194,14 @@ uint64_t zdraw_hip_command_count(void);
 uint64_t zdraw_hip_attn_fallback_count(void);
 uint64_t zdraw_hip_gpu_ns(void); /* device time summed over completed batches / blocking runs */
 
+/* Attention-kernel trace (the attention bucket of ZDRAW_KLEIN_TRACE,
+ * klein/zflux2_resident.zig:443-467): when on, each attention kernel launch is
+ * bracketed by its own HIP events on the stream it is launched on (a pre-pass
+ * kernel is outside the bracket). trace_attention_ns waits for the bracketed
+ * launches, returns their summed device time and stores their count. */
+void zdraw_hip_trace_attention(int on);
+uint64_t zdraw_hip_trace_attention_ns(uint64_t* launches);
+
 /* HIP events on a queue's stream, for measuring kernels where they run. */
 void* zdraw_hip_event_create(void);
 int zdraw_hip_event_record(void* event, void* queue);
@@ -195,9 +211,8 @@ void zdraw_hip_event_release(void* event);
 int zdraw_hip_queue_sync(void* queue);
 
 /* Measurement knob: which build of the attention kernel runs.
- * Software-pipelined kernel: 0 = 64 query rows per wave x 4 waves (default),
- * 1 = 32 rows x 8 waves, 2 = 32 rows x 4 waves (two workgroups per CU).
- * Unpipelined kernel: 3 = 32 rows x 8 waves, 4 = 32 rows x 4 waves. */
+ * 0 = 8 waves x 32 query rows per workgroup, one workgroup per CU (default);
+ * 1 = 4 waves x 32 query rows, two workgroups per CU. */
 void zdraw_hip_set_attention_variant(int variant);
 
 /* ABI drift guard (src/abi_gen.zig, runtime/abi_assert.zig:29): sizeof of the
@@ -208,7 +223,7 @@ size_t zdraw_hip_abi_sizeof(int which);
 const char* zdraw_hip_last_error(void);
 
 #define ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE 24
-#define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 208
+#define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 216
 #define ZDRAW_HIP_ABI_QK_OPERANDS_SIZE 72
 
 #ifdef __cplusplus

@@ -34,11 +34,11 @@ def test_abi_struct_sizes():
     L = hip.lib()
     # AttnParams must stay 24 bytes (runtime/abi_assert.zig:29)
     assert L.zdraw_hip_abi_sizeof(0) == 24 == C.sizeof(hip.AttnParams)
-    assert L.zdraw_hip_abi_sizeof(1) == C.sizeof(hip.AttnExt) == 208
+    assert L.zdraw_hip_abi_sizeof(1) == C.sizeof(hip.AttnExt) == 216
     assert L.zdraw_hip_abi_sizeof(2) == C.sizeof(hip.QkOperands) == 72
     text = open(os.path.join(ROOT, "include", "zdraw_hip.h")).read()
     assert "#define ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE 24" in text
-    assert "#define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 208" in text
+    assert "#define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 216" in text
     assert "#define ZDRAW_HIP_ABI_QK_OPERANDS_SIZE 72" in text
 
 

@@ -154,10 +154,12 @@ def test_config1_plumbing_through_attention_fast(ctx):
 @pytest.mark.parametrize("name", ["klein_1024", "klein_512_x4", "zimage_1024", "klein_edit_ragged"])
 @pytest.mark.parametrize("k_site", [hip.K_IN_TILE_LOAD, hip.K_PREPASS])
 @pytest.mark.parametrize("dtype", [hip.BF16, hip.F32])
-def test_small_configs_all_rows(ctx, name, k_site, dtype):
-    say(f"small config {name} k_site={k_site} dtype={dtype}")
+@pytest.mark.parametrize("bounded", [True, False])
+def test_small_configs_all_rows(ctx, name, k_site, dtype, bounded):
+    # bounded: the caller's score bound lets the kernel skip the running maximum
+    say(f"small config {name} k_site={k_site} dtype={dtype} bounded={bounded}")
     w = wl.by_name(name, seed=5, small=True)
-    res = wl.Resident(ctx, w, dtype=dtype, k_site=k_site)
+    res = wl.Resident(ctx, w, dtype=dtype, k_site=k_site, bounded=bounded)
     got = res.run()
     again = res.run()
     res.release()
@@ -184,6 +186,8 @@ def test_full_configs_sampled_rows_and_bit_stability(ctx, name, nsample):
     res.k_site = hip.K_PREPASS
     res.ext.k_site = hip.K_PREPASS
     pre = res.run()
+    res.ext.score_bound = 0.0  # running-maximum softmax
+    dyn = res.run()
     res.release()
     toks = refimpl.sample_tokens(w, nsample)
     say(f"  oracle on {len(toks)} query tokens x {w.batch} segments")
@@ -192,6 +196,8 @@ def test_full_configs_sampled_rows_and_bit_stability(ctx, name, nsample):
     say(f"  tile-load K: max abs {mx:.2e} mean abs {mean:.2e}")
     mx, mean = refimpl.check_close(pre[:, toks], want, name + " (K pre-pass)")
     say(f"  pre-pass  K: max abs {mx:.2e} mean abs {mean:.2e}")
+    mx, mean = refimpl.check_close(dyn[:, toks], want, name + " (running maximum)")
+    say(f"  running max: max abs {mx:.2e} mean abs {mean:.2e}")
     assert np.isfinite(got).all() and np.isfinite(pre).all()
     # no row left unwritten: every output row has a non-zero element
     assert (np.abs(got).max(axis=-1) > 0).all()
@@ -246,7 +252,8 @@ def test_text_row_weights_select_by_token(ctx):
     wb = [ctx.buffer(a) for a in (wq, wk, wqt, wkt)]
     cos, sin = ctx.buffer(w.rope_cos), ctx.buffer(w.rope_sin)
     ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=w.tokens, heads=w.heads, norm_q=wb[0], norm_k=wb[1],
-                    norm_added_q=wb[2], norm_added_k=wb[3], txt_rows=w.txt_len, rope_cos=cos, rope_sin=sin)
+                    norm_added_q=wb[2], norm_added_k=wb[3], txt_rows=w.txt_len, rope_cos=cos, rope_sin=sin,
+                    score_bound=host.score_bound(wq, wk, wqt, wkt))
     got = host.bf16_bits_to_f32(o.read(np.uint16, w.q.shape))[0]
     t = w.txt_len
     qn = np.concatenate([zo.klein_rms_norm_heads(w.q[0, :t], wqt), zo.klein_rms_norm_heads(w.q[0, t:], wq)])

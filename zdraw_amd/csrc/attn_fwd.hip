@@ -1,21 +1,32 @@
-// gfx950 flash-attention forward, software-pipelined form: 64 query rows per
-// wave, four waves per workgroup (256 query rows share every K/V block).
+// gfx950 flash-attention forward for zdraw's DiT joint self-attention.
 //
-// Compared with the 32-rows-per-wave kernel this one
-//   * reuses each K fragment and each V fragment for two MFMAs (two 32-query
-//     blocks per wave), halving LDS reads per FLOP;
-//   * keeps V row-major in LDS and builds the V^T operand with the transposing
-//     LDS read (ds_read_b64_tr_b16), so staging V is a plain 16-byte copy;
-//   * walks the keys in blocks of 32 through a 4-stage LDS ring and overlaps,
-//     inside one wave, the MFMAs of S(b+1) = K(b+1) Q^T and O += V(b-1)^T P(b-1)
-//     with the softmax VALU work of block b (the three are independent), one
-//     barrier per block.
-// Block order is fixed; there are no atomics; results are bit-stable.
+// What it replaces in the reference: the Metal attention kernels behind
+// zdraw_metal_run_attention* (metal/mattn_block_shader.zig:7-188, the steel
+// route metal_api.m:6685-6815) and, when K is prepared in the tile load, the
+// QK-norm + rope glue kernels that feed them (klein/zflux2_glue_shader.zig:61-122,
+// metal/mqk_shader.zig:46-97). The design is MI355X-first, not a translation:
+//
+//   * one wave owns 32 query rows; the waves of a workgroup share every K/V block;
+//   * scores are computed TRANSPOSED (S^T = K . Q^T) with v_mfma_f32_32x32x16_bf16,
+//     so every lane owns one query column: softmax reductions are in-lane plus
+//     one permlane32 swap, and the exponentiated block is already the B operand
+//     of the second MFMA (O^T = V^T . P^T): no LDS round trip for P;
+//   * K blocks sit in LDS row-major (272-byte pitch, conflict-free b128 reads);
+//     V blocks sit row-major too (320-byte pitch) and the V^T operand is built
+//     by the transposing LDS read ds_read_b64_tr_b16, so staging V is a plain copy;
+//   * RMSNorm + rope are applied to the Q rows once in the prologue and to the
+//     K rows between the global load and the LDS store of each block;
+//   * keys are walked in blocks of 32 through an LDS ring; inside one wave the
+//     MFMAs of S(b+1) = K(b+1) Q^T and O += V(b-1)^T P(b-1) are interleaved, slot
+//     by slot, with the softmax VALU work of block b (the three are independent);
+//   * global loads run two steps ahead of the LDS store that consumes them;
+//   * block order is fixed and nothing is accumulated with atomics, so the
+//     output is bit-identical from run to run.
 #include "attn_device.hpp"
 
 namespace zdraw {
 
-namespace v2 {
+namespace fwd {
 
 #ifndef ZDRAW_DIAG
 #define ZDRAW_DIAG 0 // timing experiments only: 1 no softmax VALU, 2 no MFMA, 4 no LDS fragment reads, 8 no barrier, 16 no staging
@@ -67,8 +78,14 @@ __device__ __forceinline__ s16x4 lds_read_tr(const bf16_t* p) {
 //   QB=2, NW=4: one wave per SIMD with the full 512-register budget;
 //   QB=1, NW=8: two waves per SIMD, 256 registers each;
 //   QB=1, NW=4: two workgroups per CU, each with its own LDS ring.
-template <typename TIn, int KMODE, bool MASKED, int QB, int NW>
-__global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel(const AttnArgs a) {
+//
+// BOUNDED: the caller has promised that every scaled score fits comfortably in
+// the fp32 exponent (QK-normalised operands: |q'.k'|/sqrt(D) <= sqrt(D) max|w_q| max|w_k|).
+// Softmax is shift-invariant, so the kernel then exponentiates the scores as
+// they are: no running maximum, no subtraction, no rescale of O. Otherwise the
+// lazy running maximum below is used.
+template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
+__global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(const AttnArgs a) {
     constexpr int NT = NW * 64;
     constexpr int QR = 32 * QB;       // query rows per wave
     constexpr int BQ = NW * QR;       // query rows per workgroup
@@ -105,11 +122,12 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
     const int head = bh - seg * a.heads;
     const int q0 = qb * BQ + wave * QR;
 
-    // zero the ring: the pipeline's first O update and last S update touch
-    // stages that no block has been stored to yet
+    // The pipeline's first O update multiplies P = 0 by the V stage of "block -1":
+    // that stage must hold finite numbers, so it is zeroed. (The last S update
+    // reads a K stage past the end; its result is discarded.)
     {
-        u32x4* z = reinterpret_cast<u32x4*>(smem);
-        const int n16 = (int)((size_t)NST * (KS_ELEMS + VS_ELEMS) * sizeof(bf16_t) / 16);
+        u32x4* z = reinterpret_cast<u32x4*>(Vs + (NST - 1) * VS_ELEMS);
+        constexpr int n16 = (int)(VS_ELEMS * sizeof(bf16_t) / 16);
         for (int i = tid; i < n16; i += NT) z[i] = u32x4{0u, 0u, 0u, 0u};
     }
 
@@ -166,8 +184,13 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
                 qk_apply8(a.q_mode, x[s], inv, r.w, d0, t);
             }
         }
+        // log2(e)/sqrt(D) rides on Q, so the MFMA delivers scores in the exp2 domain
 #pragma unroll
-        for (int s = 0; s < 8; s++) qf[qi][s] = __builtin_bit_cast(bf16x8, pack_bf16x8(x[s]));
+        for (int s = 0; s < 8; s++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) x[s][i] *= a.scale_log2;
+            qf[qi][s] = __builtin_bit_cast(bf16x8, pack_bf16x8(x[s]));
+        }
     }
 
     // ---- block staging: thread t owns key t/TPK of the block, CPT chunks of 8 dims of K and of V
@@ -176,46 +199,54 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
     const TIn* const kbase = reinterpret_cast<const TIn*>(a.k) + (int64_t)seg * a.k_bs + (int64_t)head * a.k_hs + lk_d0;
     const TIn* const vbase = reinterpret_cast<const TIn*>(a.v) + (int64_t)seg * a.v_bs + (int64_t)head * a.v_hs + lk_d0;
 
-    Raw8<TIn> kraw[CPT], vraw[CPT];
-    Rope8 krope[KMODE == kQkNone ? 1 : CPT];
-    QkRow krow;
+    // Two register sets alternate: a block's global loads are issued two steps
+    // before the step that moves it into LDS, so a full step of work always
+    // separates a load from its first use.
+    struct StageRegs {
+        Raw8<TIn> kraw[CPT], vraw[CPT];
+        Rope8 krope[KMODE == kQkNone ? 1 : CPT];
+        QkRow krow;
+    };
+    StageRegs sets[2];
 
     // i = position in the block list. Loads are unconditional (no branches in
     // the pipelined loop): positions past the end re-read the last block and
     // rows past the sequence re-read its last row. Neither is ever used: the
     // drained ring stages feed only discarded MFMAs, and keys past the limit
-    // are masked to -inf before the softmax.
+    // are masked to -inf before the softmax. Row offsets are 32-bit element
+    // counts (the host checks that a head's rows span less than 2^31 elements).
     const int last_row = a.tokens - 1;
-    auto stage_load = [&](int i) {
+    const unsigned k_ts32 = (unsigned)a.k_ts, v_ts32 = (unsigned)a.v_ts;
+    auto stage_load = [&](StageRegs& r, int i) __attribute__((always_inline)) {
         const int ii = i < nblk ? i : nblk - 1;
         int key = block_of(ii) * KB + lk_key;
         key = key < last_row ? key : last_row;
-        const TIn* pk = kbase + (int64_t)key * a.k_ts;
-        const TIn* pv = vbase + (int64_t)key * a.v_ts;
+        const TIn* pk = kbase + (unsigned)key * k_ts32;
+        const TIn* pv = vbase + (unsigned)key * v_ts32;
 #pragma unroll
         for (int c = 0; c < CPT; c++) {
-            kraw[c] = ld_raw8<TIn>(pk + 8 * c, true);
-            vraw[c] = ld_raw8<TIn>(pv + 8 * c, true);
+            r.kraw[c] = ld_raw8<TIn>(pk + 8 * c, true);
+            r.vraw[c] = ld_raw8<TIn>(pv + 8 * c, true);
         }
         if constexpr (KMODE != kQkNone) {
-            krow = qk_row(a.qk, KMODE, a.k_w, a.k_w_txt, seg, key, true);
+            r.krow = qk_row(a.qk, KMODE, a.k_w, a.k_w_txt, seg, key, true);
 #pragma unroll
-            for (int c = 0; c < CPT; c++) krope[c] = ld_rope8(a.qk, KMODE, krow, lk_d0 + 8 * c);
+            for (int c = 0; c < CPT; c++) r.krope[c] = ld_rope8(a.qk, KMODE, r.krow, lk_d0 + 8 * c);
         }
     };
 
-    auto stage_store = [&](int stage) {
+    auto stage_store = [&](StageRegs& r, int stage) __attribute__((always_inline)) {
         bf16_t* kdst = Ks + stage * KS_ELEMS + lk_key * KPITCH + lk_d0;
         bf16_t* vdst = Vs + stage * VS_ELEMS + lk_key * VPITCH + lk_d0;
         if constexpr (KMODE == kQkNone) {
 #pragma unroll
-            for (int c = 0; c < CPT; c++) *reinterpret_cast<u32x4*>(kdst + 8 * c) = raw_to_bf16(kraw[c]);
+            for (int c = 0; c < CPT; c++) *reinterpret_cast<u32x4*>(kdst + 8 * c) = raw_to_bf16(r.kraw[c]);
         } else {
             float x[CPT][8];
             float ss = 0.f;
 #pragma unroll
             for (int c = 0; c < CPT; c++) {
-                unpack8(kraw[c], x[c]);
+                unpack8(r.kraw[c], x[c]);
 #pragma unroll
                 for (int i = 0; i < 8; i++) ss += x[c][i] * x[c][i];
             }
@@ -223,12 +254,12 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
             const float inv = rsqrtf(ss * (1.0f / D) + a.qk.eps);
 #pragma unroll
             for (int c = 0; c < CPT; c++) {
-                qk_apply8(KMODE, x[c], inv, krow.w, lk_d0 + 8 * c, krope[c]);
+                qk_apply8(KMODE, x[c], inv, r.krow.w, lk_d0 + 8 * c, r.krope[c]);
                 *reinterpret_cast<u32x4*>(kdst + 8 * c) = pack_bf16x8(x[c]);
             }
         }
 #pragma unroll
-        for (int c = 0; c < CPT; c++) *reinterpret_cast<u32x4*>(vdst + 8 * c) = raw_to_bf16(vraw[c]);
+        for (int c = 0; c < CPT; c++) *reinterpret_cast<u32x4*>(vdst + 8 * c) = raw_to_bf16(r.vraw[c]);
     };
 
     // ---- running state
@@ -289,14 +320,14 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
     //   LDS reads for the MFMA two slots ahead | one MFMA per query block |
     //   one slice of the softmax VALU work, which runs in the MFMA's shadow.
     // Even slots extend S(b+1) = K(b+1) Q^T, odd slots add V(b-1)^T P(b-1)^T to O^T.
-    auto step = [&](int b, bool sync, f32x16 (&s_cur)[QB], f32x16 (&s_next)[QB], const bf16x8 (&p_prev)[QB][2],
+    auto step = [&](int b, StageRegs& regs, bool sync, f32x16 (&s_cur)[QB], f32x16 (&s_next)[QB], const bf16x8 (&p_prev)[QB][2],
                     bf16x8 (&p_cur)[QB][2]) __attribute__((always_inline)) {
-        // ring: block b+AHEAD (in registers since the previous step) goes to its stage,
+        // ring: block b+AHEAD (in this register set since two steps ago) goes to its stage,
         // whose previous tenant's last reader (V, NST-AHEAD-1 steps back) is at least one
-        // barrier behind; then the loads of block b+AHEAD+1 start
+        // barrier behind; then the set starts loading block b+AHEAD+2
         if (!(ZDRAW_DIAG & 16)) {
-            stage_store((b + AHEAD) & (NST - 1));
-            stage_load(b + AHEAD + 1);
+            stage_store(regs, (b + AHEAD) & (NST - 1));
+            stage_load(regs, b + AHEAD + 2);
         }
 
         const bf16_t* kt = Ks + ((b + 1) & (NST - 1)) * KS_ELEMS + l32 * KPITCH + 8 * h;
@@ -357,58 +388,81 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
         float t[QB][7], mc[QB], alpha[QB], psum[QB];
         unsigned pc[QB][8] = {}; // P as packed bf16 pairs
         bool grew = false;
-        if (ZDRAW_DIAG & 1) {
-            for (int qi = 0; qi < QB; qi++) { alpha[qi] = 1.f; p_cur[qi][0] = p_prev[qi][0]; p_cur[qi][1] = p_prev[qi][1]; }
+#pragma unroll
+        for (int qi = 0; qi < QB; qi++) {
+            mc[qi] = 0.f;
+            alpha[qi] = 1.f;
+            psum[qi] = 0.f;
         }
-        // softmax of S(b) in 16 slices (per query block)
+        if (ZDRAW_DIAG & 1) {
+            for (int qi = 0; qi < QB; qi++) { p_cur[qi][0] = p_prev[qi][0]; p_cur[qi][1] = p_prev[qi][1]; }
+        }
+        // exponentials of elements 2*pr, 2*pr+1 of this lane's 16 scores
+        auto exp_pair = [&](int qi, int pr) __attribute__((always_inline)) {
+            f32x16& sv = s_cur[qi];
+            f32x2 pp;
+            if constexpr (BOUNDED) {
+                pp[0] = __builtin_amdgcn_exp2f(sv[2 * pr]);
+                pp[1] = __builtin_amdgcn_exp2f(sv[2 * pr + 1]);
+            } else {
+                pp[0] = __builtin_amdgcn_exp2f(sv[2 * pr] - mc[qi]);
+                pp[1] = __builtin_amdgcn_exp2f(sv[2 * pr + 1] - mc[qi]);
+            }
+            psum[qi] += pp[0] + pp[1];
+            pc[qi][pr] = __builtin_bit_cast(unsigned, __builtin_convertvector(pp, bf16x2));
+            pin(psum[qi]);
+            pin(pc[qi][pr]);
+        };
+        // softmax of S(b) in 16 slices (per query block), spread so that every
+        // MFMA has about the same amount of VALU work behind it
         auto valu_slice = [&](int c) __attribute__((always_inline)) {
             if (ZDRAW_DIAG & 1) return;
-            if ((ZDRAW_DIAG & 32) && c >= 7 && c <= 10) return; // half of the exponentials
 #pragma unroll
             for (int qi = 0; qi < QB; qi++) {
                 f32x16& sv = s_cur[qi];
-                if (c == 0) {
-                    t[qi][0] = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
-                    t[qi][1] = fmaxf(fmaxf(sv[3], sv[4]), sv[5]);
-                    t[qi][2] = fmaxf(fmaxf(sv[6], sv[7]), sv[8]);
-                    t[qi][3] = fmaxf(fmaxf(sv[9], sv[10]), sv[11]);
-                } else if (c == 1) {
-                    t[qi][4] = fmaxf(fmaxf(sv[12], sv[13]), sv[14]);
-                    t[qi][5] = fmaxf(fmaxf(t[qi][0], t[qi][1]), t[qi][2]);
-                    t[qi][6] = fmaxf(fmaxf(t[qi][3], t[qi][4]), sv[15]);
-                    t[qi][0] = fmaxf(t[qi][5], t[qi][6]);
-                } else if (c == 2) {
-                    // Lazy running maximum, kept in the exp2 domain: the reference point of
-                    // the exponentials only moves when this block's maximum exceeds it by
-                    // more than kTau, so P stays within [0, 2^kTau] and O is rescaled on a
-                    // handful of blocks instead of on every new row maximum.
-                    const float mlc = pair_max(t[qi][0]) * a.scale_log2;
-                    const bool up = mlc > m_run[qi] + kTau;
-                    const float m_new = up ? mlc : m_run[qi];
-                    mc[qi] = (m_new == -INFINITY) ? 0.f : m_new;
-                    alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - mc[qi]);
-                    grew |= up;
-                    m_run[qi] = m_new;
-                    psum[qi] = 0.f;
-                    pin(mc[qi]);
-                    pin(alpha[qi]);
-                } else if (c <= 10) {
-                    const int e = 2 * (c - 3); // elements e, e+1 of 16
-                    f32x2 pp;
-                    pp[0] = __builtin_amdgcn_exp2f(sv[e] * a.scale_log2 - mc[qi]);
-                    pp[1] = __builtin_amdgcn_exp2f(sv[e + 1] * a.scale_log2 - mc[qi]);
-                    const bf16x2 pr = __builtin_convertvector(pp, bf16x2);
-                    // the denominator sums the same bf16-rounded weights the MFMA multiplies by
-                    psum[qi] = __builtin_amdgcn_fdot2_f32_bf16(pr, bf16x2{(bf16_t)1.0f, (bf16_t)1.0f}, psum[qi], false);
-                    pc[qi][e >> 1] = __builtin_bit_cast(unsigned, pr);
-                    pin(psum[qi]);
-                    pin(pc[qi][e >> 1]);
-                } else if (c == 12) {
+                if constexpr (BOUNDED) {
+                    if ((c & 1) == 0) exp_pair(qi, c >> 1);
+                    if (c == 15) {
+                        l_run[qi] += psum[qi];
+                        pin(l_run[qi]);
+                    }
+                } else {
+                    if (c == 0) {
+                        t[qi][0] = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
+                        t[qi][1] = fmaxf(fmaxf(sv[3], sv[4]), sv[5]);
+                        t[qi][2] = fmaxf(fmaxf(sv[6], sv[7]), sv[8]);
+                        t[qi][3] = fmaxf(fmaxf(sv[9], sv[10]), sv[11]);
+                    } else if (c == 1) {
+                        t[qi][4] = fmaxf(fmaxf(sv[12], sv[13]), sv[14]);
+                        t[qi][5] = fmaxf(fmaxf(t[qi][0], t[qi][1]), t[qi][2]);
+                        t[qi][6] = fmaxf(fmaxf(t[qi][3], t[qi][4]), sv[15]);
+                        t[qi][0] = fmaxf(t[qi][5], t[qi][6]);
+                    } else if (c == 2) {
+                        // Lazy running maximum (exp2 domain): the reference point of the
+                        // exponentials only moves when this block's maximum exceeds it by
+                        // more than kTau, so P stays within [0, 2^kTau] and O is rescaled on
+                        // a handful of blocks instead of on every new row maximum.
+                        const float mlc = pair_max(t[qi][0]);
+                        const bool up = mlc > m_run[qi] + kTau;
+                        const float m_new = up ? mlc : m_run[qi];
+                        mc[qi] = (m_new == -INFINITY) ? 0.f : m_new;
+                        alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - mc[qi]);
+                        grew |= up;
+                        m_run[qi] = m_new;
+                        pin(mc[qi]);
+                        pin(alpha[qi]);
+                    } else if (c <= 14) {
+                        // pairs on slices 3,4, 6,7, 9,10, 12,13
+                        const int r = c - 3;
+                        if (r % 3 != 2) exp_pair(qi, (r / 3) * 2 + (r % 3));
+                    } else {
+                        l_run[qi] = l_run[qi] * alpha[qi] + psum[qi];
+                        pin(l_run[qi]);
+                    }
+                }
+                if (c == 15) {
                     p_cur[qi][0] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][0], pc[qi][1], pc[qi][2], pc[qi][3]});
                     p_cur[qi][1] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][4], pc[qi][5], pc[qi][6], pc[qi][7]});
-                } else if (c == 14) {
-                    l_run[qi] = l_run[qi] * alpha[qi] + psum[qi];
-                    pin(l_run[qi]);
                 }
             }
         };
@@ -426,7 +480,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
         }
 
         // O is relative to m(b-1) here; move it to m(b) before block b's update lands
-        if (__any(grew)) {
+        if (!BOUNDED && __any(grew)) {
 #pragma unroll
             for (int qi = 0; qi < QB; qi++)
 #pragma unroll
@@ -438,14 +492,15 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
     };
 
     if (nblk > 0) {
-        // prologue: blocks 0 .. AHEAD-1 into the ring, block AHEAD in flight
-        stage_load(0);
+        // prologue: blocks 0 .. AHEAD-1 into the ring, blocks AHEAD and AHEAD+1 in flight
+        stage_load(sets[0], 0);
         __syncthreads(); // ring zeroing complete
 #pragma unroll
         for (int i = 0; i < AHEAD; i++) {
-            stage_store(i);
-            stage_load(i + 1);
+            stage_store(sets[0], i);
+            stage_load(sets[0], i + 1);
         }
+        stage_load(sets[1], AHEAD + 1);
         __syncthreads();
 
         f32x16 s_a[QB], s_b[QB];
@@ -462,11 +517,11 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
         // 8-stage ring only the second step of a trip ends in a barrier
         int b = 0;
         for (; b + 1 < nblk; b += 2) {
-            step(b, NST != 8, s_a, s_b, p_a, p_b);
-            step(b + 1, true, s_b, s_a, p_b, p_a);
+            step(b, sets[0], NST != 8, s_a, s_b, p_a, p_b);
+            step(b + 1, sets[1], true, s_b, s_a, p_b, p_a);
         }
         if (b < nblk) {
-            step(b, true, s_a, s_b, p_a, p_b);
+            step(b, sets[0], true, s_a, s_b, p_a, p_b);
             pv_block((nblk - 1) & (NST - 1), p_b);
         } else {
             pv_block((nblk - 1) & (NST - 1), p_a);
@@ -508,41 +563,47 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_v2_kernel
     }
 }
 
-template <typename TIn, int KMODE, bool MASKED, int QB, int NW>
+template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
 static hipError_t launch_one(const AttnArgs& a, hipStream_t stream) {
     const int64_t nwg = (int64_t)a.nqb * a.heads * a.batch;
     if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
-    attn_fwd_v2_kernel<TIn, KMODE, MASKED, QB, NW>
+    attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
         <<<dim3((unsigned)nwg), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
     return hipGetLastError();
 }
 
-template <typename TIn, bool MASKED, int QB, int NW>
+template <typename TIn, bool MASKED, bool BOUNDED, int QB, int NW>
 static hipError_t launch_kmode(const AttnArgs& a, int k_mode, hipStream_t stream) {
     switch (k_mode) {
-    case kQkNone: return launch_one<TIn, kQkNone, MASKED, QB, NW>(a, stream);
-    case kQkKlein: return launch_one<TIn, kQkKlein, MASKED, QB, NW>(a, stream);
-    case kQkZimage: return launch_one<TIn, kQkZimage, MASKED, QB, NW>(a, stream);
+    case kQkNone: return launch_one<TIn, kQkNone, MASKED, BOUNDED, QB, NW>(a, stream);
+    case kQkKlein: return launch_one<TIn, kQkKlein, MASKED, BOUNDED, QB, NW>(a, stream);
+    case kQkZimage: return launch_one<TIn, kQkZimage, MASKED, BOUNDED, QB, NW>(a, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
-template <int QB, int NW>
-static hipError_t launch_shape(const AttnArgs& a, int in_dtype, int k_mode, hipStream_t stream) {
+template <typename TIn, int QB, int NW>
+static hipError_t launch_flags(const AttnArgs& a, int k_mode, hipStream_t stream) {
     // the masked build is only needed when some key of some block is excluded
     const bool masked = a.key_pad != nullptr || (a.key_limit % KB) != 0;
-    if (in_dtype == kF32)
-        return masked ? launch_kmode<float, true, QB, NW>(a, k_mode, stream)
-                      : launch_kmode<float, false, QB, NW>(a, k_mode, stream);
-    if (in_dtype == kBF16)
-        return masked ? launch_kmode<bf16_t, true, QB, NW>(a, k_mode, stream)
-                      : launch_kmode<bf16_t, false, QB, NW>(a, k_mode, stream);
+    const bool bounded = a.bounded != 0;
+    if (masked)
+        return bounded ? launch_kmode<TIn, true, true, QB, NW>(a, k_mode, stream)
+                       : launch_kmode<TIn, true, false, QB, NW>(a, k_mode, stream);
+    return bounded ? launch_kmode<TIn, false, true, QB, NW>(a, k_mode, stream)
+                   : launch_kmode<TIn, false, false, QB, NW>(a, k_mode, stream);
+}
+
+template <int QB, int NW>
+static hipError_t launch_shape(const AttnArgs& a, int in_dtype, int k_mode, hipStream_t stream) {
+    if (in_dtype == kF32) return launch_flags<float, QB, NW>(a, k_mode, stream);
+    if (in_dtype == kBF16) return launch_flags<bf16_t, QB, NW>(a, k_mode, stream);
     return hipErrorInvalidValue;
 }
 
-template <typename TIn, int KMODE, bool MASKED, int QB, int NW>
+template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
 static hipError_t raise_lds() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_v2_kernel<TIn, KMODE, MASKED, QB, NW>),
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(ring_stages(QB, NW)));
 }
 
@@ -550,35 +611,34 @@ template <int QB, int NW>
 static hipError_t raise_shape() {
     hipError_t e;
 #define ZD_RAISE(T, M) \
-    if ((e = raise_lds<T, M, false, QB, NW>()) != hipSuccess) return e; \
-    if ((e = raise_lds<T, M, true, QB, NW>()) != hipSuccess) return e;
+    if ((e = raise_lds<T, M, false, false, QB, NW>()) != hipSuccess) return e; \
+    if ((e = raise_lds<T, M, true, false, QB, NW>()) != hipSuccess) return e; \
+    if ((e = raise_lds<T, M, false, true, QB, NW>()) != hipSuccess) return e; \
+    if ((e = raise_lds<T, M, true, true, QB, NW>()) != hipSuccess) return e;
     ZD_RAISE(float, kQkNone) ZD_RAISE(float, kQkKlein) ZD_RAISE(float, kQkZimage)
     ZD_RAISE(bf16_t, kQkNone) ZD_RAISE(bf16_t, kQkKlein) ZD_RAISE(bf16_t, kQkZimage)
 #undef ZD_RAISE
     return hipSuccess;
 }
 
-} // namespace v2
+} // namespace fwd
 
-// shape: 0 = 2 query blocks x 4 waves, 1 = 1 x 8, 2 = 1 x 4
-int attention_v2_block_rows(int shape) { return shape == 0 ? 256 : (shape == 1 ? 256 : 128); }
-int attention_v2_key_block() { return v2::KB; }
-int attention_v2_max_tokens() { return v2::MAX_BLOCKS * v2::KB; }
+int attention_block_rows(int shape) { return shape == 1 ? 128 : 256; }
+int attention_key_block() { return fwd::KB; }
+int attention_max_tokens() { return fwd::MAX_BLOCKS * fwd::KB; }
 
-hipError_t launch_attention_v2(const AttnArgs& a, int in_dtype, int k_mode, int shape, hipStream_t stream) {
+hipError_t launch_attention(const AttnArgs& a, int in_dtype, int k_mode, int shape, hipStream_t stream) {
     switch (shape) {
-    case 0: return v2::launch_shape<2, 4>(a, in_dtype, k_mode, stream);
-    case 1: return v2::launch_shape<1, 8>(a, in_dtype, k_mode, stream);
-    case 2: return v2::launch_shape<1, 4>(a, in_dtype, k_mode, stream);
+    case 0: return fwd::launch_shape<1, 8>(a, in_dtype, k_mode, stream);
+    case 1: return fwd::launch_shape<1, 4>(a, in_dtype, k_mode, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
-hipError_t attention_v2_setup() {
+hipError_t attention_setup() {
     hipError_t e;
-    if ((e = v2::raise_shape<2, 4>()) != hipSuccess) return e;
-    if ((e = v2::raise_shape<1, 8>()) != hipSuccess) return e;
-    if ((e = v2::raise_shape<1, 4>()) != hipSuccess) return e;
+    if ((e = fwd::raise_shape<1, 8>()) != hipSuccess) return e;
+    if ((e = fwd::raise_shape<1, 4>()) != hipSuccess) return e;
     return hipSuccess;
 }
 

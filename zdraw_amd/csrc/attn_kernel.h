@@ -8,8 +8,6 @@
 namespace zdraw {
 
 constexpr int kHeadDim = 128;      // the only head width the MFMA kernel is built for
-constexpr int kKeyTile = 64;       // keys per LDS tile
-constexpr int kMaxKeyTiles = 4096; // key-tile list capacity in LDS (tokens <= 262144)
 
 enum QkMode : int {
     kQkNone = 0,   // operands are used as given
@@ -54,6 +52,8 @@ struct AttnArgs {
     int32_t q_mode;     // QkMode applied to Q rows at load
     int32_t out_dtype;  // kF32 or kBF16
     float scale_log2;   // log2(e) / sqrt(head_dim)
+    int32_t bounded;    // 1: scaled scores are known to fit the fp32 exponent with room to spare
+    int32_t pad1;
     QkOps qk;
     // QK-norm weights (f32[128]); *_txt used for tokens < qk.txt_rows when non-null
     const float* q_w;
@@ -81,25 +81,16 @@ struct PrepArgs {
     const float* w_txt;
 };
 
-// LDS bytes the attention kernel needs (dynamic shared memory).
-size_t attention_lds_bytes();
-// Query rows per workgroup for a wave count (4 or 8).
-int attention_block_rows(int nwaves);
-
+// Kernel shape: 0 = 8 waves x 32 query rows (one workgroup per CU, 8-stage LDS
+// ring), 1 = 4 waves x 32 query rows (two workgroups per CU, 4-stage rings).
+int attention_block_rows(int shape);
+int attention_key_block();
+int attention_max_tokens();
 // Launch one attention forward. in_dtype is kF32 or kBF16; k_mode is the
-// QkMode applied to K rows inside the K-tile load. Returns a hipError_t.
-hipError_t launch_attention(const AttnArgs& args, int in_dtype, int k_mode, int nwaves,
-                            hipStream_t stream);
+// QkMode applied to K rows inside the K-block load. Returns a hipError_t.
+hipError_t launch_attention(const AttnArgs& args, int in_dtype, int k_mode, int shape, hipStream_t stream);
 hipError_t launch_qk_prepass(const PrepArgs& args, int in_dtype, hipStream_t stream);
 // One-time per-device setup (raises the dynamic LDS limit on every instantiation).
 hipError_t attention_setup();
-
-// The software-pipelined kernel (64 query rows per wave, 4 waves, 32-key blocks).
-// shape: 0 = two 32-query blocks per wave x 4 waves, 1 = one x 8 waves, 2 = one x 4 waves
-int attention_v2_block_rows(int shape);
-int attention_v2_key_block();
-int attention_v2_max_tokens();
-hipError_t launch_attention_v2(const AttnArgs& args, int in_dtype, int k_mode, int shape, hipStream_t stream);
-hipError_t attention_v2_setup();
 
 } // namespace zdraw

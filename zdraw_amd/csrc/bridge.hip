@@ -17,6 +17,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <vector>
 
 using namespace zdraw;
 
@@ -55,8 +56,19 @@ uint64_t g_dispatch = 0;
 uint64_t g_command = 0;
 uint64_t g_fallback = 0;
 uint64_t g_gpu_ns = 0;
-int g_variant = 0; // 0..2: pipelined kernel shapes (2x4, 1x8, 1x4 query blocks x waves); 3, 4: unpipelined kernel, 8 / 4 waves
+int g_variant = 0; // kernel shape: 0 = 8 waves per workgroup, 1 = 4 waves (two workgroups per CU)
 bool g_setup_done = false;
+
+// Attention-kernel trace (the reference's ZDRAW_KLEIN_TRACE attention bucket,
+// klein/zflux2_resident.zig:443-467): when on, every attention launch is
+// bracketed by its own pair of events on the launch stream.
+bool g_trace = false;
+struct TracePair {
+    hipEvent_t a, b;
+};
+std::vector<TracePair> g_trace_open;
+uint64_t g_trace_ns = 0;
+uint64_t g_trace_launches = 0;
 
 thread_local char g_err[512] = "";
 
@@ -111,6 +123,10 @@ const char* check_operand(const Operand& o, uint32_t dtype, uint32_t batch, uint
         snprintf(why, sizeof(why), "%s: device pointer not 16-byte aligned", name);
         return why;
     }
+    if ((uint64_t)(tokens - 1) * o.ts + kHeadDim >= (1ull << 31) || o.ts >= (1ull << 31)) {
+        snprintf(why, sizeof(why), "%s: one head's rows span 2^31 elements or more", name);
+        return why;
+    }
     if (o.ts < kHeadDim && tokens > 1) {
         snprintf(why, sizeof(why), "%s: token stride smaller than head_dim", name);
         return why;
@@ -154,7 +170,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     if (p->causal != 0) return unavailable("causal attention");
     if (p->kv_heads != p->heads) return unavailable("grouped-query attention");
     if (x->batch == 0) return invalid("batch == 0");
-    const uint64_t max_tokens = g_variant <= 2 ? (uint64_t)attention_v2_max_tokens() : (uint64_t)kMaxKeyTiles * kKeyTile;
+    const uint64_t max_tokens = (uint64_t)attention_max_tokens();
     if ((uint64_t)p->tokens > max_tokens) return unavailable("too many tokens");
     if ((x->in_dtype != ZDRAW_HIP_F32 && x->in_dtype != ZDRAW_HIP_BF16) ||
         (x->out_dtype != ZDRAW_HIP_F32 && x->out_dtype != ZDRAW_HIP_BF16))
@@ -185,11 +201,15 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     a.heads = (int32_t)p->heads;
     a.batch = (int32_t)x->batch;
     a.key_limit = (int32_t)((p->valid != 0 && p->valid < p->tokens) ? p->valid : p->tokens);
-    const int rows = g_variant <= 2 ? attention_v2_block_rows(g_variant) : attention_block_rows(g_variant == 3 ? 8 : 4);
+    const int rows = attention_block_rows(g_variant);
     a.nqb = (int32_t)((p->tokens + rows - 1) / rows);
     a.q_mode = (int32_t)x->qk_mode;
     a.out_dtype = (int32_t)x->out_dtype;
     a.scale_log2 = 1.4426950408889634f / sqrtf((float)kHeadDim);
+    // exp2 of a scaled score must stay far from the fp32 exponent limits: 2^64 times
+    // tokens (<= 2^15) times |v| still fits, 2^-64 does not underflow
+    if (!(x->score_bound >= 0.0f)) return invalid("score_bound");
+    a.bounded = (x->score_bound > 0.0f && x->score_bound * 1.4426950408889634f <= 64.0f) ? 1 : 0;
     if ((int64_t)a.nqb * a.heads * a.batch > 0x7fffffffLL) return unavailable("grid too large");
 
     const uint64_t rows_needed = (uint64_t)(x->batch - 1) * x->rope_batch_rows + p->tokens;
@@ -284,7 +304,6 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
 int enqueue(const FusedPlan& plan, hipStream_t stream) {
     if (!g_setup_done) {
         hipError_t e = attention_setup();
-        if (e == hipSuccess) e = attention_v2_setup();
         if (e != hipSuccess) {
             set_err("attention_setup: %s", hipGetErrorString(e));
             return ZDRAW_HIP_ERR_HANDLE;
@@ -299,11 +318,17 @@ int enqueue(const FusedPlan& plan, hipStream_t stream) {
         }
         g_dispatch++;
     }
-    hipError_t e = g_variant <= 2 ? launch_attention_v2(plan.args, plan.in_dtype, plan.k_mode, g_variant, stream)
-                                  : launch_attention(plan.args, plan.in_dtype, plan.k_mode, g_variant == 3 ? 8 : 4, stream);
+    TracePair tp{nullptr, nullptr};
+    if (g_trace && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
+        (void)hipEventRecord(tp.a, stream);
+    hipError_t e = launch_attention(plan.args, plan.in_dtype, plan.k_mode, g_variant, stream);
     if (e != hipSuccess) {
         set_err("attention launch: %s", hipGetErrorString(e));
         return ZDRAW_HIP_ERR_HANDLE;
+    }
+    if (tp.a && tp.b) {
+        (void)hipEventRecord(tp.b, stream);
+        g_trace_open.push_back(tp);
     }
     g_dispatch++;
     return ZDRAW_HIP_OK;
@@ -485,7 +510,7 @@ void zdraw_hip_release_pipeline(void* pipeline) { delete static_cast<Pipeline*>(
 size_t zdraw_hip_pipeline_threads(void* pipeline) {
     Pipeline* p = static_cast<Pipeline*>(pipeline);
     if (!p) return 0;
-    return p->kind == 0 ? ((g_variant == 1 || g_variant == 3) ? 512 : 256) : 256;
+    return p->kind == 0 ? (g_variant == 0 ? 512 : 256) : 256;
 }
 
 // ---------------------------------------------------------------- attention
@@ -675,7 +700,11 @@ void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes) {
 }
 
 // --------------------------------------------------------- counters, timing
-void zdraw_hip_metrics_reset(void) { g_dispatch = g_command = g_fallback = g_gpu_ns = 0; }
+void zdraw_hip_metrics_reset(void) {
+    (void)zdraw_hip_trace_attention_ns(nullptr);
+    g_dispatch = g_command = g_fallback = g_gpu_ns = 0;
+    g_trace_ns = g_trace_launches = 0;
+}
 uint64_t zdraw_hip_dispatch_count(void) { return g_dispatch; }
 uint64_t zdraw_hip_command_count(void) { return g_command; }
 uint64_t zdraw_hip_attn_fallback_count(void) { return g_fallback; }
@@ -717,7 +746,25 @@ int zdraw_hip_queue_sync(void* queue) {
     return e == hipSuccess ? ZDRAW_HIP_OK : hip_fail(e, "queue sync");
 }
 
-void zdraw_hip_set_attention_variant(int variant) { g_variant = (variant >= 0 && variant <= 4) ? variant : 0; }
+void zdraw_hip_trace_attention(int on) { g_trace = on != 0; }
+
+uint64_t zdraw_hip_trace_attention_ns(uint64_t* launches) {
+    // fold every finished pair into the totals (waits for pairs still in flight)
+    for (TracePair& tp : g_trace_open) {
+        float ms = 0.f;
+        if (hipEventSynchronize(tp.b) == hipSuccess && hipEventElapsedTime(&ms, tp.a, tp.b) == hipSuccess) {
+            g_trace_ns += (uint64_t)((double)ms * 1e6);
+            g_trace_launches++;
+        }
+        (void)hipEventDestroy(tp.a);
+        (void)hipEventDestroy(tp.b);
+    }
+    g_trace_open.clear();
+    if (launches) *launches = g_trace_launches;
+    return g_trace_ns;
+}
+
+void zdraw_hip_set_attention_variant(int variant) { g_variant = variant == 1 ? 1 : 0; }
 
 size_t zdraw_hip_abi_sizeof(int which) {
     switch (which) {

@@ -31,6 +31,7 @@ class AttnExt(C.Structure):
         ("zimage_base", C.c_uint64 * 3), ("zimage_dims", C.c_uint32 * 3),
         ("batch", C.c_uint32), ("in_dtype", C.c_uint32), ("out_dtype", C.c_uint32),
         ("qk_mode", C.c_uint32), ("k_site", C.c_uint32), ("txt_rows", C.c_uint32), ("eps", C.c_float),
+        ("score_bound", C.c_float), ("reserved", C.c_uint32),
     ]
 
 
@@ -73,6 +74,8 @@ SYMBOLS = {
     "zdraw_hip_command_count": (_u64, []),
     "zdraw_hip_attn_fallback_count": (_u64, []),
     "zdraw_hip_gpu_ns": (_u64, []),
+    "zdraw_hip_trace_attention": (None, [_int]),
+    "zdraw_hip_trace_attention_ns": (_u64, [C.POINTER(C.c_uint64)]),
     "zdraw_hip_event_create": (_vp, []),
     "zdraw_hip_event_record": (_int, [_vp, _vp]),
     "zdraw_hip_event_sync": (_int, [_vp]),

@@ -92,7 +92,8 @@ class _Klein(C.Structure):
                 ("norm_q", C.c_void_p), ("norm_k", C.c_void_p),
                 ("norm_added_q", C.c_void_p), ("norm_added_k", C.c_void_p),
                 ("rope_cos", C.c_void_p), ("rope_sin", C.c_void_p), ("rope_per_segment", C.c_bool),
-                ("key_pad", C.c_void_p), ("out_row_stride", C.c_size_t), ("k_site", C.c_uint32)]
+                ("key_pad", C.c_void_p), ("out_row_stride", C.c_size_t), ("k_site", C.c_uint32),
+                ("score_bound", C.c_float)]
 
 
 class _Zimage(C.Structure):
@@ -101,7 +102,7 @@ class _Zimage(C.Structure):
                 ("tokens", C.c_size_t), ("heads", C.c_size_t),
                 ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("pos", C.c_void_p), ("rope_pairs", C.c_void_p),
                 ("dims", C.c_size_t * 3), ("bases", C.c_size_t * 3), ("norm_eps", C.c_float),
-                ("k_site", C.c_uint32)]
+                ("k_site", C.c_uint32), ("score_bound", C.c_float)]
 
 
 class _RopeCache(C.Structure):
@@ -152,6 +153,8 @@ def lib():
         L.zh_joint_klein.argtypes = [vp, C.POINTER(_Klein)]
         L.zh_joint_zimage.restype = C.c_int
         L.zh_joint_zimage.argtypes = [vp, C.POINTER(_Zimage)]
+        L.zh_score_bound.restype = C.c_float
+        L.zh_score_bound.argtypes = [_fp, _fp, _fp, _fp]
         L.zh_sizeof.restype = sz
         L.zh_sizeof.argtypes = [C.c_int]
         assert L.zh_sizeof(0) == C.sizeof(_ZhConfig)
@@ -287,18 +290,19 @@ class Context:
     def joint_klein(self, q, k, v, o, *, tokens, heads, nb=1, in_dtype=hip.BF16, out_dtype=hip.BF16,
                     norm_q, norm_k, norm_added_q=None, norm_added_k=None, txt_rows=0,
                     rope_cos, rope_sin, rope_per_segment=False, key_pad=None,
-                    out_row_stride=0, k_site=hip.K_IN_TILE_LOAD):
+                    out_row_stride=0, k_site=hip.K_IN_TILE_LOAD, score_bound=0.0):
         h = lambda b: b.handle if b is not None else None
         c = _Klein(h(q), h(k), h(v), h(o), in_dtype, out_dtype, tokens, heads, nb, txt_rows,
                    h(norm_q), h(norm_k), h(norm_added_q), h(norm_added_k), h(rope_cos), h(rope_sin),
-                   rope_per_segment, h(key_pad), out_row_stride, k_site)
+                   rope_per_segment, h(key_pad), out_row_stride, k_site, score_bound)
         _raise(lib().zh_joint_klein(self._ptr, C.byref(c)))
 
     def joint_zimage(self, q, k, v, o, *, tokens, heads, in_dtype=hip.BF16, out_dtype=hip.BF16,
-                     q_norm, k_norm, pos, rope_pairs, dims, bases, norm_eps, k_site=hip.K_IN_TILE_LOAD):
+                     q_norm, k_norm, pos, rope_pairs, dims, bases, norm_eps, k_site=hip.K_IN_TILE_LOAD,
+                     score_bound=0.0):
         c = _Zimage(q.handle, k.handle, v.handle, o.handle, in_dtype, out_dtype, tokens, heads,
                     q_norm.handle, k_norm.handle, pos.handle, rope_pairs.handle,
-                    (C.c_size_t * 3)(*dims), (C.c_size_t * 3)(*bases), norm_eps, k_site)
+                    (C.c_size_t * 3)(*dims), (C.c_size_t * 3)(*bases), norm_eps, k_site, score_bound)
         _raise(lib().zh_joint_zimage(self._ptr, C.byref(c)))
 
     def qk_run(self, q_buf, k_buf, q_weight, k_weight, pos, rope_values, dims, lens, *, tokens, heads,
@@ -379,3 +383,14 @@ def zimage_sequence_positions(grid_h, grid_w, cap_tokens):
     pos = np.zeros((total, 3), np.uintp)
     _raise(L.zh_zimage_sequence_positions(pos.ctypes.data_as(_sp), total, grid_h, grid_w, cap_tokens))
     return pos
+
+
+def score_bound(w_q, w_k, w_q_txt=None, w_k_txt=None) -> float:
+    """joint::scoreBound: bound on |q'.k'|/sqrt(128) for RMS-normalised, rotated operands."""
+    def ptr(w):
+        if w is None:
+            return None
+        return _f(np.ascontiguousarray(w, np.float32))
+    arrs = [None if w is None else np.ascontiguousarray(w, np.float32) for w in (w_q, w_k, w_q_txt, w_k_txt)]
+    ptrs = [None if a is None else _f(a) for a in arrs]
+    return float(lib().zh_score_bound(*ptrs))

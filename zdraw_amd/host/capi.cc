@@ -106,6 +106,10 @@ int zh_qk_run(void* ctx, void* q_h, void* k_h, const float* q_weight, const floa
 int zh_joint_klein(void* ctx, const joint::Klein* c) { return (int)joint::run(static_cast<hattn::Context*>(ctx), *c); }
 int zh_joint_zimage(void* ctx, const joint::Zimage* c) { return (int)joint::run(static_cast<hattn::Context*>(ctx), *c); }
 
+float zh_score_bound(const float* wq, const float* wk, const float* wqt, const float* wkt) {
+    return joint::scoreBound(wq, wk, wqt, wkt);
+}
+
 size_t zh_sizeof(int which) {
     switch (which) {
     case 0: return sizeof(ZhConfig);

@@ -76,6 +76,23 @@ Error run(hattn::Context* ctx, void* q_h, void* k_h, const float* q_weight, cons
 
 namespace joint {
 
+float scoreBound(const float* w_q, const float* w_k, const float* w_q_txt, const float* w_k_txt) {
+    auto amax = [](const float* w) {
+        float m = 0.f;
+        if (w)
+            for (size_t i = 0; i < hattn::flash_head_dim; i++) {
+                const float v = w[i] < 0 ? -w[i] : w[i];
+                m = v > m ? v : m;
+            }
+        return m;
+    };
+    const float mq = amax(w_q) > amax(w_q_txt) ? amax(w_q) : amax(w_q_txt);
+    const float mk = amax(w_k) > amax(w_k_txt) ? amax(w_k) : amax(w_k_txt);
+    // |q'| <= sqrt(128) mq, |k'| <= sqrt(128) mk, divided by sqrt(128); 2% slack for
+    // the rounding of the normalisation and of the bf16 operands
+    return 11.313708498984761f * mq * mk * 1.02f;
+}
+
 static void fill_strides(uint64_t* s, size_t tokens, size_t row_stride, size_t nb) {
     s[0] = nb > 1 ? (uint64_t)tokens * row_stride : 0;
     s[1] = row_stride;
@@ -107,6 +124,7 @@ Error run(hattn::Context* ctx, const Klein& c) {
     x.eps = 1e-6f; // klein/zflux2.zig:70 (rms_eps)
     x.rope_batch_rows = c.rope_per_segment ? c.tokens : 0;
     x.mask_batch_bytes = c.key_pad ? c.tokens : 0;
+    x.score_bound = c.score_bound;
     ZdrawHipQkOperands ops;
     memset(&ops, 0, sizeof(ops));
     ops.q_weight = c.norm_q;
@@ -141,6 +159,7 @@ Error run(hattn::Context* ctx, const Zimage& c) {
     x.qk_mode = ZDRAW_HIP_QK_ZIMAGE;
     x.k_site = (uint32_t)c.k_site;
     x.eps = c.norm_eps;
+    x.score_bound = c.score_bound;
     for (int a = 0; a < 3; a++) {
         x.zimage_dims[a] = (uint32_t)c.dims[a];
         x.zimage_base[a] = c.bases[a];

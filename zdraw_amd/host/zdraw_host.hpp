@@ -51,7 +51,7 @@ using CpuRun = int (*)(float* out, size_t out_len, const float* q, size_t q_len,
 
 namespace hattn {
 
-constexpr size_t max_tokens = 262144;   // key-tile list capacity of the kernel (mattn.zig:15 is 6144 for `rows`)
+constexpr size_t max_tokens = 32768;    // key-block list capacity of the kernel (mattn.zig:15 is 6144 for `rows`)
 constexpr size_t flash_head_dim = 128;  // mattn.zig:16
 
 // mattn.zig:19. Only `block` (the bf16-MFMA flash kernel) exists on gfx950.
@@ -160,8 +160,15 @@ struct Klein {
     void* key_pad;                       // u8 [nb][tokens] or null
     size_t out_row_stride;               // elements between output token rows; 0 = heads*128
     KSite k_site;
+    float score_bound;                   // see scoreBound(); 0 = unknown (running-maximum softmax)
 };
 Error run(hattn::Context* ctx, const Klein& c);
+
+// Upper bound on |q'.k'| / sqrt(128) after RMSNorm with the given weights and a
+// rope that rotates pairs (both table builders of the reference do): each
+// normalised row has norm <= sqrt(128) * max|w|. Pass null for weight sets that
+// are not in use. Valid only when the rope tables are rotations.
+float scoreBound(const float* w_q, const float* w_k, const float* w_q_txt, const float* w_k_txt);
 
 // One Z-Image single-stream attention call (zimage/zattn.zig:45-82 after the
 // projections): q, k, v, o are [tokens][heads*128].
@@ -178,6 +185,7 @@ struct Zimage {
     size_t bases[3];
     float norm_eps;
     KSite k_site;
+    float score_bound;                   // see scoreBound(); 0 = unknown
 };
 Error run(hattn::Context* ctx, const Zimage& c);
 

@@ -132,7 +132,7 @@ class Resident:
     """A workload's operands uploaded once; `launch()` enqueues one pass of the
     hot path (inputs already in HBM), `run()` also waits and reads O back."""
 
-    def __init__(self, ctx: host.Context, w: Workload, dtype=hip.BF16, k_site=hip.K_IN_TILE_LOAD):
+    def __init__(self, ctx: host.Context, w: Workload, dtype=hip.BF16, k_site=hip.K_IN_TILE_LOAD, bounded=True):
         self.ctx, self.w, self.dtype, self.k_site = ctx, w, dtype, k_site
         conv = host.f32_to_bf16_bits if dtype == hip.BF16 else (lambda a: np.ascontiguousarray(a, np.float32))
         self.q = ctx.buffer(conv(w.q))
@@ -173,6 +173,9 @@ class Resident:
             for a in range(3):
                 x.zimage_dims[a] = ZIMAGE_DIMS[a]
                 x.zimage_base[a] = w.rope_bases[a]
+        if w.kind != "plain" and bounded:
+            # unit norm weights: the normalised rows have norm sqrt(128), rope rotates
+            x.score_bound = host.score_bound(ones, ones)
         if self.key_pad is not None:
             self.ops.key_pad = self.key_pad.handle
             x.mask_batch_bytes = w.tokens
