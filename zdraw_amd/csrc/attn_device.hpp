@@ -43,6 +43,26 @@ __device__ __forceinline__ Raw8<T> ld_raw8(const T* p, bool ok) {
     return x;
 }
 
+// The same chunk through a buffer resource: the address is a wave-uniform
+// descriptor (base in scalar registers) + a per-thread byte offset + a uniform
+// byte offset, so a loop that walks blocks spends no vector ALU work on it.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    // word 3: 32-bit data format, raw (unstrided) addressing
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+template <typename T>
+__device__ __forceinline__ Raw8<T> ld_raw8_buf(rsrc_t rsrc, unsigned thread_off, unsigned uniform_off) {
+    Raw8<T> x;
+    if constexpr (std::is_same<T, float>::value) {
+        x.a = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)thread_off, (int)uniform_off, 0));
+        x.b = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(thread_off + 16), (int)uniform_off, 0));
+    } else {
+        x.r = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)thread_off, (int)uniform_off, 0));
+    }
+    return x;
+}
+
 __device__ __forceinline__ void unpack8(const Raw8<float>& r, float (&x)[8]) {
 #pragma unroll
     for (int i = 0; i < 4; i++) { x[i] = r.a[i]; x[4 + i] = r.b[i]; }

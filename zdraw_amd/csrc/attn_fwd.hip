@@ -28,11 +28,17 @@ namespace zdraw {
 
 namespace fwd {
 
-#ifndef ZDRAW_DIAG
-#define ZDRAW_DIAG 0 // timing experiments only: 1 no softmax VALU, 2 no MFMA, 4 no LDS fragment reads, 8 no barrier, 16 no staging
-#endif
 #ifndef ZDRAW_LDS_LOOKAHEAD
 #define ZDRAW_LDS_LOOKAHEAD 4
+#endif
+#ifndef ZDRAW_MFMA_PRIO
+#define ZDRAW_MFMA_PRIO 1
+#endif
+#ifndef ZDRAW_READ_BATCH
+#define ZDRAW_READ_BATCH 2
+#endif
+#ifndef ZDRAW_STORE_SLOT
+#define ZDRAW_STORE_SLOT 1
 #endif
 
 constexpr int KB = 32;            // keys per block
@@ -92,8 +98,12 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     constexpr int CPT = 512 / NT;     // 8-element chunks of K (and of V) per thread per block
     constexpr int TPK = 16 / CPT;     // threads sharing one key row
     constexpr int NST = ring_stages(QB, NW);
-    constexpr int AHEAD = NST == 8 ? 3 : 2;   // a block is stored AHEAD steps before S needs its K
+    constexpr bool XSTEP = NST == 8;          // fragment reads run ahead across step boundaries
+    constexpr int AHEAD = NST == 8 ? 4 : 2;   // a block is stored AHEAD steps before S needs its K
     constexpr int LA = ZDRAW_LDS_LOOKAHEAD;   // slots between an LDS fragment read and its MFMA
+    constexpr int RB = ZDRAW_READ_BATCH;      // slots whose reads are issued together (divides 16 and LA)
+    constexpr int MFMA_PRIO = ZDRAW_MFMA_PRIO; // wave priority while an MFMA is being issued
+    constexpr int STORE_SLOT = ZDRAW_STORE_SLOT; // slot after which the ring store is issued
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* const Ks = reinterpret_cast<bf16_t*>(smem);
     bf16_t* const Vs = Ks + NST * KS_ELEMS;
@@ -153,9 +163,10 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             if (lane == 0) s_nblocks = count;
         }
         __syncthreads();
-        nblk = s_nblocks;
+        nblk = __builtin_amdgcn_readfirstlane(s_nblocks);
     }
-    auto block_of = [&](int i) -> int { return (MASKED && kp) ? (int)blocks[i] : i; };
+    // wave-uniform by construction; readfirstlane lets the compiler keep it in scalar registers
+    auto block_of = [&](int i) -> int { return (MASKED && kp) ? __builtin_amdgcn_readfirstlane((int)blocks[i]) : i; };
 
     // ---- Q rows -> B-operand registers: qf[qi][s], lane: query 32*qi + l32, dims 16s + 8h .. +7
     bf16x8 qf[QB][8];
@@ -196,8 +207,24 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // ---- block staging: thread t owns key t/TPK of the block, CPT chunks of 8 dims of K and of V
     const int lk_key = tid / TPK;
     const int lk_d0 = (tid % TPK) * CPT * 8;
-    const TIn* const kbase = reinterpret_cast<const TIn*>(a.k) + (int64_t)seg * a.k_bs + (int64_t)head * a.k_hs + lk_d0;
-    const TIn* const vbase = reinterpret_cast<const TIn*>(a.v) + (int64_t)seg * a.v_bs + (int64_t)head * a.v_hs + lk_d0;
+    // Addresses are a wave-uniform buffer descriptor (segment, head) + a uniform
+    // byte offset (key block) + a 32-bit per-thread byte offset that never
+    // changes (row within the block, column): the loop spends no vector ALU
+    // work on them. The host checks that a head's rows span less than 4 GiB.
+    const unsigned k_span = ((unsigned)(a.tokens - 1) * (unsigned)a.k_ts + D) * (unsigned)sizeof(TIn);
+    const unsigned v_span = ((unsigned)(a.tokens - 1) * (unsigned)a.v_ts + D) * (unsigned)sizeof(TIn);
+    const rsrc_t k_rsrc = make_rsrc(reinterpret_cast<const TIn*>(a.k) + (int64_t)seg * a.k_bs + (int64_t)head * a.k_hs, k_span);
+    const rsrc_t v_rsrc = make_rsrc(reinterpret_cast<const TIn*>(a.v) + (int64_t)seg * a.v_bs + (int64_t)head * a.v_hs, v_span);
+    const unsigned k_blk_bytes = (unsigned)a.k_ts * (unsigned)(KB * sizeof(TIn));
+    const unsigned v_blk_bytes = (unsigned)a.v_ts * (unsigned)(KB * sizeof(TIn));
+    const unsigned k_off = ((unsigned)lk_key * (unsigned)a.k_ts + (unsigned)lk_d0) * (unsigned)sizeof(TIn);
+    const unsigned v_off = ((unsigned)lk_key * (unsigned)a.v_ts + (unsigned)lk_d0) * (unsigned)sizeof(TIn);
+    // the block that holds the last row: its rows past the sequence re-read the last row
+    const int last_row = a.tokens - 1;
+    const int last_blk = last_row / KB;
+    const int lk_tail = min(lk_key, last_row - last_blk * KB);
+    const unsigned k_off_tail = ((unsigned)lk_tail * (unsigned)a.k_ts + (unsigned)lk_d0) * (unsigned)sizeof(TIn);
+    const unsigned v_off_tail = ((unsigned)lk_tail * (unsigned)a.v_ts + (unsigned)lk_d0) * (unsigned)sizeof(TIn);
 
     // Two register sets alternate: a block's global loads are issued two steps
     // before the step that moves it into LDS, so a full step of work always
@@ -210,25 +237,29 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     StageRegs sets[2];
 
     // i = position in the block list. Loads are unconditional (no branches in
-    // the pipelined loop): positions past the end re-read the last block and
-    // rows past the sequence re-read its last row. Neither is ever used: the
-    // drained ring stages feed only discarded MFMAs, and keys past the limit
-    // are masked to -inf before the softmax. Row offsets are 32-bit element
-    // counts (the host checks that a head's rows span less than 2^31 elements).
-    const int last_row = a.tokens - 1;
-    const unsigned k_ts32 = (unsigned)a.k_ts, v_ts32 = (unsigned)a.v_ts;
+    // the pipelined loop): positions past the end re-read the last block.
+    // Neither those nor the rows past the sequence are ever used: the drained
+    // ring stages feed only discarded MFMAs, and keys past the limit are
+    // masked to -inf before the softmax. (The unmasked build only runs when
+    // every block is full, so it needs no tail offsets.)
     auto stage_load = [&](StageRegs& r, int i) __attribute__((always_inline)) {
         const int ii = i < nblk ? i : nblk - 1;
-        int key = block_of(ii) * KB + lk_key;
-        key = key < last_row ? key : last_row;
-        const TIn* pk = kbase + (unsigned)key * k_ts32;
-        const TIn* pv = vbase + (unsigned)key * v_ts32;
+        const int blk = block_of(ii);
+        unsigned ko = k_off, vo = v_off;
+        if constexpr (MASKED) {
+            const bool tail = blk >= last_blk; // wave-uniform
+            ko = tail ? k_off_tail : k_off;
+            vo = tail ? v_off_tail : v_off;
+        }
+        const unsigned kb = (unsigned)blk * k_blk_bytes, vb = (unsigned)blk * v_blk_bytes;
 #pragma unroll
         for (int c = 0; c < CPT; c++) {
-            r.kraw[c] = ld_raw8<TIn>(pk + 8 * c, true);
-            r.vraw[c] = ld_raw8<TIn>(pv + 8 * c, true);
+            r.kraw[c] = ld_raw8_buf<TIn>(k_rsrc, ko + (unsigned)(8 * c * sizeof(TIn)), kb);
+            r.vraw[c] = ld_raw8_buf<TIn>(v_rsrc, vo + (unsigned)(8 * c * sizeof(TIn)), vb);
         }
         if constexpr (KMODE != kQkNone) {
+            int key = blk * KB + lk_key;
+            key = key < last_row ? key : last_row;
             r.krow = qk_row(a.qk, KMODE, a.k_w, a.k_w_txt, seg, key, true);
 #pragma unroll
             for (int c = 0; c < CPT; c++) r.krope[c] = ld_rope8(a.qk, KMODE, r.krow, lk_d0 + 8 * c);
@@ -314,42 +345,37 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         }
     };
 
+    // Fragment registers of the software pipeline; they live across steps because the
+    // first reads of a step are issued at the end of the step before it.
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    bf16x8 kf[8];
+    s16x4 vlo[8], vhi[8];
+    // LDS fragment read for slot `slot` of step `bb`: even slots read K(bb+1) dims
+    // 16*(slot/2).., odd slots read the V(bb-1) patch for output block (slot/2)%4, keys 16*(slot/8)..
+    auto frag_read = [&](int bb, int slot) __attribute__((always_inline)) {
+        if (slot & 1) {
+            const bf16_t* vt = Vs + ((bb + NST - 1) & (NST - 1)) * VS_ELEMS + (4 * h + tr_row) * VPITCH + tr_col;
+            const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
+            vlo[idx] = lds_read_tr(vt + (16 * kb) * VPITCH + 32 * blk);
+            vhi[idx] = lds_read_tr(vt + (16 * kb + 8) * VPITCH + 32 * blk);
+        } else {
+            const bf16_t* kt = Ks + ((bb + 1) & (NST - 1)) * KS_ELEMS + l32 * KPITCH + 8 * h;
+            kf[slot >> 1] = *reinterpret_cast<const bf16x8*>(kt + 16 * (slot >> 1));
+        }
+    };
+
     // One pipeline step for list position b: consumes S(b) and P(b-1),
     // produces S(b+1) and P(b). The three streams are independent, so the
     // step is laid out by hand as 16 slots, each fenced from the next:
-    //   LDS reads for the MFMA two slots ahead | one MFMA per query block |
+    //   LDS reads for the MFMA LA slots ahead | one MFMA per query block |
     //   one slice of the softmax VALU work, which runs in the MFMA's shadow.
     // Even slots extend S(b+1) = K(b+1) Q^T, odd slots add V(b-1)^T P(b-1)^T to O^T.
+    // With the 8-stage ring the reads for the first LA slots of step b+1 are
+    // issued in the last LA slots of step b, so no step starts by waiting on LDS.
     auto step = [&](int b, StageRegs& regs, bool sync, f32x16 (&s_cur)[QB], f32x16 (&s_next)[QB], const bf16x8 (&p_prev)[QB][2],
                     bf16x8 (&p_cur)[QB][2]) __attribute__((always_inline)) {
-        // ring: block b+AHEAD (in this register set since two steps ago) goes to its stage,
-        // whose previous tenant's last reader (V, NST-AHEAD-1 steps back) is at least one
-        // barrier behind; then the set starts loading block b+AHEAD+2
-        if (!(ZDRAW_DIAG & 16)) {
-            stage_store(regs, (b + AHEAD) & (NST - 1));
-            stage_load(regs, b + AHEAD + 2);
-        }
-
-        const bf16_t* kt = Ks + ((b + 1) & (NST - 1)) * KS_ELEMS + l32 * KPITCH + 8 * h;
-        const bf16_t* vt = Vs + ((b + NST - 1) & (NST - 1)) * VS_ELEMS + (4 * h + tr_row) * VPITCH + tr_col;
-        typedef short s16x8 __attribute__((ext_vector_type(8)));
-        bf16x8 kf[8];
-        s16x4 vlo[8], vhi[8];
-        if (ZDRAW_DIAG & 4) {
-            for (int i = 0; i < 8; i++) { kf[i] = qf[0][i]; vlo[i] = s16x4{1, 2, 3, 4}; vhi[i] = vlo[i]; }
-        }
-        auto read_slot = [&](int slot) __attribute__((always_inline)) {
-            if (ZDRAW_DIAG & 4) return;
-            if (slot & 1) {
-                const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
-                vlo[idx] = lds_read_tr(vt + (16 * kb) * VPITCH + 32 * blk);
-                vhi[idx] = lds_read_tr(vt + (16 * kb + 8) * VPITCH + 32 * blk);
-            } else {
-                kf[slot >> 1] = *reinterpret_cast<const bf16x8*>(kt + 16 * (slot >> 1));
-            }
-        };
         auto mfma_slot = [&](int slot) __attribute__((always_inline)) {
-            if (ZDRAW_DIAG & 2) return;
+            if (MFMA_PRIO) __builtin_amdgcn_s_setprio(MFMA_PRIO);
             if (slot & 1) {
                 const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
                 const bf16x8 vf =
@@ -363,6 +389,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 for (int qi = 0; qi < QB; qi++)
                     s_next[qi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[qi][st], s_next[qi], 0, 0, 0);
             }
+            if (MFMA_PRIO) __builtin_amdgcn_s_setprio(0);
         };
 
         if constexpr (MASKED) {
@@ -394,9 +421,6 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             alpha[qi] = 1.f;
             psum[qi] = 0.f;
         }
-        if (ZDRAW_DIAG & 1) {
-            for (int qi = 0; qi < QB; qi++) { p_cur[qi][0] = p_prev[qi][0]; p_cur[qi][1] = p_prev[qi][1]; }
-        }
         // exponentials of elements 2*pr, 2*pr+1 of this lane's 16 scores
         auto exp_pair = [&](int qi, int pr) __attribute__((always_inline)) {
             f32x16& sv = s_cur[qi];
@@ -416,7 +440,6 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         // softmax of S(b) in 16 slices (per query block), spread so that every
         // MFMA has about the same amount of VALU work behind it
         auto valu_slice = [&](int c) __attribute__((always_inline)) {
-            if (ZDRAW_DIAG & 1) return;
 #pragma unroll
             for (int qi = 0; qi < QB; qi++) {
                 f32x16& sv = s_cur[qi];
@@ -467,15 +490,29 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             }
         };
 
-        // LDS reads run LA slots ahead of the MFMA that consumes them
+        if constexpr (!XSTEP) {
 #pragma unroll
-        for (int g = 0; g < LA; g++) read_slot(g);
-        __builtin_amdgcn_sched_barrier(0);
+            for (int g = 0; g < LA; g++) frag_read(b, g);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int g = 0; g < 16; g++) {
-            if (g + LA < 16) read_slot(g + LA);
+            // reads are issued RB slots' worth at a time, so one wait covers RB MFMAs
+            if (g % RB == 0) {
+#pragma unroll
+                for (int j = 0; j < RB; j++) {
+                    const int slot = g + LA + j;
+                    if (slot < 16) frag_read(b, slot);
+                    else if constexpr (XSTEP) frag_read(b + 1, slot - 16);
+                }
+            }
             mfma_slot(g);
             valu_slice(g);
+            // ring: block b+AHEAD (in this register set since two steps ago) goes to its stage,
+            // whose previous tenant's last reader (V, NST-AHEAD-1 steps back) is at least one
+            // barrier behind; then the set starts loading block b+AHEAD+2
+            if (g == STORE_SLOT) stage_store(regs, (b + AHEAD) & (NST - 1));
+            if (g == STORE_SLOT + 1) stage_load(regs, b + AHEAD + 2);
             __builtin_amdgcn_sched_barrier(0);
         }
 
@@ -488,19 +525,33 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
                     for (int j = 0; j < 16; j++) oacc[qi][blk][j] *= alpha[qi];
         }
-        if (sync && !(ZDRAW_DIAG & 8)) __syncthreads();
+        if (sync) {
+            if constexpr (XSTEP) {
+                // Only the next step's first fragment reads are outstanding here and they
+                // touch stages no one writes before the next barrier. LDS operations of a
+                // wave complete in order and every read of this step has been consumed, so
+                // this step's ring writes are complete: the bare barrier orders them.
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            } else {
+                __syncthreads();
+            }
+        }
     };
 
     if (nblk > 0) {
         // prologue: blocks 0 .. AHEAD-1 into the ring, blocks AHEAD and AHEAD+1 in flight
-        stage_load(sets[0], 0);
-        __syncthreads(); // ring zeroing complete
+        {
+            StageRegs pre[AHEAD];
 #pragma unroll
-        for (int i = 0; i < AHEAD; i++) {
-            stage_store(sets[0], i);
-            stage_load(sets[0], i + 1);
+            for (int i = 0; i < AHEAD; i++) stage_load(pre[i], i);
+            stage_load(sets[0], AHEAD);
+            stage_load(sets[1], AHEAD + 1);
+            __syncthreads(); // ring zeroing complete
+#pragma unroll
+            for (int i = 0; i < AHEAD; i++) stage_store(pre[i], i);
         }
-        stage_load(sets[1], AHEAD + 1);
         __syncthreads();
 
         f32x16 s_a[QB], s_b[QB];
@@ -512,6 +563,10 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
                 for (int j = 0; j < 8; j++) p_a[qi][kb][j] = (bf16_t)0.0f;
         qk_block(0, s_a);
+        if constexpr (XSTEP) {
+#pragma unroll
+            for (int g = 0; g < LA; g++) frag_read(0, g);
+        }
 
         // two steps per trip so the S and P buffers swap roles without copies; with the
         // 8-stage ring only the second step of a trip ends in a barrier
@@ -623,7 +678,7 @@ static hipError_t raise_shape() {
 
 } // namespace fwd
 
-int attention_block_rows(int shape) { return shape == 1 ? 128 : 256; }
+int attention_block_rows(int shape) { return shape == 1 ? 128 : 256; } // shape 2: 4 waves x 64 rows
 int attention_key_block() { return fwd::KB; }
 int attention_max_tokens() { return fwd::MAX_BLOCKS * fwd::KB; }
 
@@ -631,6 +686,7 @@ hipError_t launch_attention(const AttnArgs& a, int in_dtype, int k_mode, int sha
     switch (shape) {
     case 0: return fwd::launch_shape<1, 8>(a, in_dtype, k_mode, stream);
     case 1: return fwd::launch_shape<1, 4>(a, in_dtype, k_mode, stream);
+    case 2: return fwd::launch_shape<2, 4>(a, in_dtype, k_mode, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -639,6 +695,7 @@ hipError_t attention_setup() {
     hipError_t e;
     if ((e = fwd::raise_shape<1, 8>()) != hipSuccess) return e;
     if ((e = fwd::raise_shape<1, 4>()) != hipSuccess) return e;
+    if ((e = fwd::raise_shape<2, 4>()) != hipSuccess) return e;
     return hipSuccess;
 }
 

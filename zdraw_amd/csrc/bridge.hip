@@ -123,8 +123,9 @@ const char* check_operand(const Operand& o, uint32_t dtype, uint32_t batch, uint
         snprintf(why, sizeof(why), "%s: device pointer not 16-byte aligned", name);
         return why;
     }
-    if ((uint64_t)(tokens - 1) * o.ts + kHeadDim >= (1ull << 31) || o.ts >= (1ull << 31)) {
-        snprintf(why, sizeof(why), "%s: one head's rows span 2^31 elements or more", name);
+    // the kernel addresses the rows of one head with 32-bit byte offsets from the head's first row
+    if (o.ts >= (1ull << 31) || ((uint64_t)(tokens - 1) * o.ts + kHeadDim) * es >= (1ull << 32)) {
+        snprintf(why, sizeof(why), "%s: one head's rows span 4 GiB or more", name);
         return why;
     }
     if (o.ts < kHeadDim && tokens > 1) {
@@ -764,7 +765,7 @@ uint64_t zdraw_hip_trace_attention_ns(uint64_t* launches) {
     return g_trace_ns;
 }
 
-void zdraw_hip_set_attention_variant(int variant) { g_variant = variant == 1 ? 1 : 0; }
+void zdraw_hip_set_attention_variant(int variant) { g_variant = (variant >= 0 && variant <= 2) ? variant : 0; }
 
 size_t zdraw_hip_abi_sizeof(int which) {
     switch (which) {
