@@ -89,7 +89,7 @@ typedef struct ZdrawHipAttnExt {
     uint32_t zimage_dims[3];   /* Z-Image axis widths, sum = head_dim */
     uint32_t batch;            /* independent segments, >= 1 */
     uint32_t in_dtype;         /* ZDRAW_HIP_F32 or ZDRAW_HIP_BF16 */
-    uint32_t out_dtype;        /* ZDRAW_HIP_F32 or ZDRAW_HIP_BF16 */
+    uint32_t out_dtype;        /* ZDRAW_HIP_F32, ZDRAW_HIP_F16 or ZDRAW_HIP_BF16 */
     uint32_t qk_mode;          /* ZDRAW_HIP_QK_* */
     uint32_t k_site;           /* ZDRAW_HIP_K_IN_TILE_LOAD or ZDRAW_HIP_K_PREPASS */
     uint32_t txt_rows;         /* tokens < txt_rows use the *_txt weights (Klein double block) */

@@ -266,6 +266,48 @@ def test_text_row_weights_select_by_token(ctx):
         b.release()
 
 
+@pytest.mark.parametrize("out_dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("k_site", [hip.K_IN_TILE_LOAD, hip.K_PREPASS])
+def test_resident_contract_f32_in_concat_operand_out(ctx, out_dtype, k_site):
+    # The Klein resident layout (klein/zflux2_resident.zig:1407-1411, 2023-2063):
+    # un-normalised f32 token-major q, k, v [nb*tokens][hidden] for nb segments
+    # [txt_0|img_0|txt_1|img_1], per-stream norm weights, one rope table shared by
+    # the segments; O lands in the first `hidden` columns of the single block's
+    # half/bf16 concat operand, whose rows are hidden + inner wide. The columns
+    # to the right of O belong to the MLP half and must stay untouched.
+    w = wl.by_name("klein_512_x4", seed=11, small=True)
+    nb, tokens, heads = 2, w.tokens, w.heads
+    hidden, inner = heads * 128, 3 * heads * 128
+    rng = np.random.default_rng(5)
+    wq, wk, wqt, wkt = (1.0 + 0.2 * rng.standard_normal(128).astype(np.float32) for _ in range(4))
+    q, k, v = w.q[:nb], w.k[:nb], w.v[:nb]
+    bufs = [ctx.buffer(np.ascontiguousarray(a, np.float32)) for a in (q, k, v)]
+    pitch = hidden + inner
+    sentinel = np.full((nb * tokens, pitch), 0x3C00 if out_dtype == "f16" else 0x3F80, np.uint16)  # 1.0 everywhere
+    o = ctx.buffer(sentinel)
+    wb = [ctx.buffer(a) for a in (wq, wk, wqt, wkt)]
+    cos, sin = ctx.buffer(w.rope_cos), ctx.buffer(w.rope_sin)
+    ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=tokens, heads=heads, nb=nb, in_dtype=hip.F32,
+                    out_dtype=hip.F16 if out_dtype == "f16" else hip.BF16, norm_q=wb[0], norm_k=wb[1],
+                    norm_added_q=wb[2], norm_added_k=wb[3], txt_rows=w.txt_len, rope_cos=cos, rope_sin=sin,
+                    out_row_stride=pitch, k_site=k_site, score_bound=host.score_bound(wq, wk, wqt, wkt))
+    raw = o.read(np.uint16, (nb * tokens, pitch))
+    assert np.array_equal(raw[:, hidden:], sentinel[:, hidden:]), "columns outside O were written"
+    bits = np.ascontiguousarray(raw[:, :hidden])
+    got = (bits.view(np.float16).astype(np.float32) if out_dtype == "f16" else host.bf16_bits_to_f32(bits))
+    got = got.reshape(nb, tokens, heads, 128)
+    t = w.txt_len
+    c2, s2 = zo.klein_build_rope_ref(w.grid[0], w.grid[1], theta=w.theta, txt_len=t)
+    for b in range(nb):
+        qn = np.concatenate([zo.klein_rms_norm_heads(q[b, :t], wqt), zo.klein_rms_norm_heads(q[b, t:], wq)])
+        kn = np.concatenate([zo.klein_rms_norm_heads(k[b, :t], wkt), zo.klein_rms_norm_heads(k[b, t:], wk)])
+        qn, kn = zo.klein_apply_rope(qn, c2, s2), zo.klein_apply_rope(kn, c2, s2)
+        want = zo.attention_run(qn, kn, v[b], zo.Config(tokens, heads, heads, 128))
+        refimpl.check_close(got[b], want, f"resident segment {b} {out_dtype}")
+    for x in bufs + wb + [o, cos, sin]:
+        x.release()
+
+
 # ----------------------------------------------------------- C-ABI level behaviour
 def test_batch_offsets_address_image_segments(ctx):
     # zdraw_metal_run_attention_enc_off: one call per segment at byte offsets

@@ -19,7 +19,9 @@
 //   * keys are walked in blocks of 32 through an LDS ring; inside one wave the
 //     MFMAs of S(b+1) = K(b+1) Q^T and O += V(b-1)^T P(b-1) are interleaved, slot
 //     by slot, with the softmax VALU work of block b (the three are independent);
-//   * global loads run two steps ahead of the LDS store that consumes them;
+//   * K/V blocks are fetched with buffer loads (descriptor + scalar block offset,
+//     no per-step address arithmetic) two steps ahead of the LDS store that
+//     consumes them; LDS fragment reads run ahead across step boundaries;
 //   * block order is fixed and nothing is accumulated with atomics, so the
 //     output is bit-identical from run to run.
 #include "attn_device.hpp"
@@ -28,17 +30,19 @@ namespace zdraw {
 
 namespace fwd {
 
+// Schedule constants of the pipelined step. They can be overridden on the
+// compiler command line to measure alternatives; the defaults are the measured best.
 #ifndef ZDRAW_LDS_LOOKAHEAD
-#define ZDRAW_LDS_LOOKAHEAD 4
-#endif
-#ifndef ZDRAW_MFMA_PRIO
-#define ZDRAW_MFMA_PRIO 1
+#define ZDRAW_LDS_LOOKAHEAD 4 // slots between an LDS fragment read and the MFMA that consumes it
 #endif
 #ifndef ZDRAW_READ_BATCH
-#define ZDRAW_READ_BATCH 2
+#define ZDRAW_READ_BATCH 2    // slots whose fragment reads are issued together (one wait per batch)
+#endif
+#ifndef ZDRAW_MFMA_PRIO
+#define ZDRAW_MFMA_PRIO 1     // wave priority while an MFMA is issued (0 = leave it alone)
 #endif
 #ifndef ZDRAW_STORE_SLOT
-#define ZDRAW_STORE_SLOT 1
+#define ZDRAW_STORE_SLOT 1    // slot after which a step moves its staged block into the ring
 #endif
 
 constexpr int KB = 32;            // keys per block
@@ -49,10 +53,11 @@ constexpr int VS_ELEMS = KB * VPITCH;
 constexpr int MAX_BLOCKS = 1024;  // key-block list capacity (tokens <= 32768)
 constexpr float kTau = 8.0f;             // log2 headroom of the lazy softmax maximum
 
-// Ring depth: 8 stages when one workgroup owns the CU (blocks are stored three
+// Ring depth: 8 stages when one workgroup owns the CU (blocks are stored four
 // steps ahead of their first use, so one barrier per two steps orders every
-// write against its readers), 4 stages when two workgroups share the CU's LDS
-// (stored two steps ahead, one barrier per step).
+// write against its readers, including the reads a step issues for the next
+// one), 4 stages when two workgroups share the CU's LDS (stored two steps
+// ahead, one barrier per step).
 constexpr int ring_stages(int qb, int nw) { return (qb == 2 || nw == 8) ? 8 : 4; }
 constexpr size_t lds_bytes(int nst) {
     return (size_t)nst * (KS_ELEMS + VS_ELEMS) * sizeof(bf16_t) + (size_t)MAX_BLOCKS * sizeof(unsigned short);
@@ -80,10 +85,11 @@ __device__ __forceinline__ s16x4 lds_read_tr(const bf16_t* p) {
         (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(p)));
 }
 
-// QB = 32-query blocks per wave (1 or 2), NW = waves per workgroup.
-//   QB=2, NW=4: one wave per SIMD with the full 512-register budget;
-//   QB=1, NW=8: two waves per SIMD, 256 registers each;
+// QB = 32-query blocks per wave, NW = waves per workgroup. Built shapes:
+//   QB=1, NW=8: two waves per SIMD, 256 registers each (default);
 //   QB=1, NW=4: two workgroups per CU, each with its own LDS ring.
+// (QB=2, NW=4, one 64-query wave per SIMD, halves the LDS reads per MFMA but
+// measured 8 % slower: one wave per SIMD cannot hide its own waits.)
 //
 // BOUNDED: the caller has promised that every scaled score fits comfortably in
 // the fp32 exponent (QK-normalised operands: |q'.k'|/sqrt(D) <= sqrt(D) max|w_q| max|w_k|).
@@ -602,6 +608,18 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                         for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
                         *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
                     }
+            } else if (a.out_dtype == kF16) {
+                typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+                _Float16* op = reinterpret_cast<_Float16*>(a.o) + off;
+#pragma unroll
+                for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        f32x4 v;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
+                        *reinterpret_cast<f16x4*>(op + 32 * blk + 8 * i + 4 * h) = __builtin_convertvector(v, f16x4);
+                    }
             } else {
                 bf16_t* op = reinterpret_cast<bf16_t*>(a.o) + off;
 #pragma unroll
@@ -678,7 +696,7 @@ static hipError_t raise_shape() {
 
 } // namespace fwd
 
-int attention_block_rows(int shape) { return shape == 1 ? 128 : 256; } // shape 2: 4 waves x 64 rows
+int attention_block_rows(int shape) { return shape == 1 ? 128 : 256; }
 int attention_key_block() { return fwd::KB; }
 int attention_max_tokens() { return fwd::MAX_BLOCKS * fwd::KB; }
 
@@ -686,7 +704,6 @@ hipError_t launch_attention(const AttnArgs& a, int in_dtype, int k_mode, int sha
     switch (shape) {
     case 0: return fwd::launch_shape<1, 8>(a, in_dtype, k_mode, stream);
     case 1: return fwd::launch_shape<1, 4>(a, in_dtype, k_mode, stream);
-    case 2: return fwd::launch_shape<2, 4>(a, in_dtype, k_mode, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -695,7 +712,6 @@ hipError_t attention_setup() {
     hipError_t e;
     if ((e = fwd::raise_shape<1, 8>()) != hipSuccess) return e;
     if ((e = fwd::raise_shape<1, 4>()) != hipSuccess) return e;
-    if ((e = fwd::raise_shape<2, 4>()) != hipSuccess) return e;
     return hipSuccess;
 }
 

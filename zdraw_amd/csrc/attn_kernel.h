@@ -50,7 +50,7 @@ struct AttnArgs {
     int32_t key_limit;  // keys >= key_limit are excluded (min(S, valid))
     int32_t nqb;        // query blocks per (segment, head)
     int32_t q_mode;     // QkMode applied to Q rows at load
-    int32_t out_dtype;  // kF32 or kBF16
+    int32_t out_dtype;  // kF32, kF16 or kBF16
     float scale_log2;   // log2(e) / sqrt(head_dim)
     int32_t bounded;    // 1: scaled scores are known to fit the fp32 exponent with room to spare
     int32_t pad1;

@@ -174,7 +174,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     const uint64_t max_tokens = (uint64_t)attention_max_tokens();
     if ((uint64_t)p->tokens > max_tokens) return unavailable("too many tokens");
     if ((x->in_dtype != ZDRAW_HIP_F32 && x->in_dtype != ZDRAW_HIP_BF16) ||
-        (x->out_dtype != ZDRAW_HIP_F32 && x->out_dtype != ZDRAW_HIP_BF16))
+        (x->out_dtype != ZDRAW_HIP_F32 && x->out_dtype != ZDRAW_HIP_BF16 && x->out_dtype != ZDRAW_HIP_F16))
         return unavailable("activation dtype");
     if (x->qk_mode > ZDRAW_HIP_QK_ZIMAGE) return invalid("qk_mode");
 
@@ -765,7 +765,7 @@ uint64_t zdraw_hip_trace_attention_ns(uint64_t* launches) {
     return g_trace_ns;
 }
 
-void zdraw_hip_set_attention_variant(int variant) { g_variant = (variant >= 0 && variant <= 2) ? variant : 0; }
+void zdraw_hip_set_attention_variant(int variant) { g_variant = variant == 1 ? 1 : 0; }
 
 size_t zdraw_hip_abi_sizeof(int which) {
     switch (which) {
