@@ -112,6 +112,7 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="kernel shape: 0 = 8 waves, 1 = 4 waves x 2 workgroups")
     ap.add_argument("--dynamic-max", action="store_true", help="withhold the score bound (running-maximum softmax)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only sustained-rate probe")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a known-size kernel to scale "
                          "the profiler's FETCH_SIZE / WRITE_SIZE counters against)")
@@ -135,9 +136,38 @@ def main():
     timed_region(L, ctx, res, max(args.warmup, 1))
     wall, kern_ms = timed_region(L, ctx, res, args.steps)
 
+    # one more launch with the clock probe on: the shader clock the kernel really ran at
+    L.zdraw_hip_clock_probe(1)
+    timed_region(L, ctx, res, 20)
+    L.zdraw_hip_clock_probe(0)
+    cyc = (C.c_uint64 * 4096)()
+    ref = (C.c_uint64 * 4096)()
+    nwg = L.zdraw_hip_clock_probe_read(cyc, ref, 4096)
+    clock = None
+    if nwg:
+        cy = np.array(cyc[:nwg], dtype=np.float64)
+        rt = np.array(ref[:nwg], dtype=np.float64)
+        ghz = cy / np.maximum(rt, 1.0) * 0.1  # reference counter ticks at 100 MHz
+        first = slice(0, min(nwg, 256))      # workgroups resident while every CU is busy
+        clock = {
+            "workgroups": int(nwg),
+            "cycles_per_workgroup_median": float(np.median(cy)),
+            "ghz_all_cus_busy_median": float(np.median(ghz[first])),
+            "ghz_last_round_median": float(np.median(ghz[256:])) if nwg > 256 else None,
+            "us_per_workgroup_all_cus_busy_median": float(np.median(rt[first]) / 100.0),
+        }
+
     out = res.read_output()
     if not np.isfinite(out).all():
         raise RuntimeError("non-finite output")
+
+    # what a loop of nothing but MFMAs sustains on this board, for the roofline's context
+    mfma_only = {}
+    if not args.no_mfma_probe:
+        for label, rnd in (("normal_operands", 1), ("constant_operands", 0)):
+            t = C.c_double(0.0)
+            if L.zdraw_hip_mfma_probe(rnd, 600, C.byref(t)) == 0:
+                mfma_only[label] = t.value
 
     # the other K site, for the record (short, untimed by the driver's clock)
     other = "tile" if args.k_site == "prepass" else "prepass"
@@ -186,6 +216,8 @@ def main():
             "traffic": traffic,
             "kernel": "attn_fwd_kernel",
             "kernel_ms": kern_ms,
+            "shader_clock": clock,
+            "mfma_only_sustained_tflops": mfma_only or None,
         },
     }
     res.release()

@@ -202,6 +202,22 @@ uint64_t zdraw_hip_gpu_ns(void); /* device time summed over completed batches / 
 void zdraw_hip_trace_attention(int on);
 uint64_t zdraw_hip_trace_attention_ns(uint64_t* launches);
 
+/* Clock probe (no reference counterpart: measurement). While on, every workgroup
+ * of an attention launch records how long it ran in shader-clock cycles and in
+ * ticks of the fixed 100 MHz reference counter; cycles / ticks x 0.1 is the clock
+ * in GHz that the kernel really ran at (under load the power limit sets it).
+ * clock_probe_read waits for the last probed launch and copies the first
+ * `capacity` workgroups' figures (in launch order); it returns how many. */
+void zdraw_hip_clock_probe(int on);
+size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t capacity);
+
+/* Sustained rate of a loop of nothing but bf16 MFMAs (no reference counterpart:
+ * measurement), run back to back for about `milliseconds` on the current device;
+ * the last launch's TFLOP/s is returned. random_operands != 0 feeds normally
+ * distributed operands, 0 feeds constants: the board's power limit makes the
+ * first markedly slower, and it is the ceiling that applies to real data. */
+int zdraw_hip_mfma_probe(int random_operands, int milliseconds, double* tflops);
+
 /* HIP events on a queue's stream, for measuring kernels where they run. */
 void* zdraw_hip_event_create(void);
 int zdraw_hip_event_record(void* event, void* queue);

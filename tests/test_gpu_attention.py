@@ -385,6 +385,24 @@ def test_abi_return_codes(ctx):
     small.release()
 
 
+def test_clock_probe_reports_every_workgroup_and_leaves_results_alone(ctx):
+    L = hip.lib()
+    w = wl.by_name("klein_1024", seed=2, small=True)
+    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_PREPASS)
+    base = res.run()
+    L.zdraw_hip_clock_probe(1)
+    probed = res.run()
+    L.zdraw_hip_clock_probe(0)
+    assert np.array_equal(base.view(np.uint32), probed.view(np.uint32))
+    cyc, ref = (C.c_uint64 * 64)(), (C.c_uint64 * 64)()
+    n = L.zdraw_hip_clock_probe_read(cyc, ref, 64)
+    rows = 256  # query rows per workgroup of the default kernel shape
+    assert n == min(64, -(-w.tokens // rows) * w.heads * w.batch)
+    ghz = np.array(cyc[:n], float) / np.array(ref[:n], float) * 0.1
+    assert (np.array(cyc[:n]) > 0).all() and (ghz > 0.05).all() and (ghz < 4.0).all()
+    res.release()
+
+
 def test_scratch_is_grow_only_and_filled(ctx):
     L = hip.lib()
     a = L.zdraw_hip_attn_scratch(ctx.device, 4, 4096)

@@ -116,6 +116,11 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     unsigned short* const blocks = reinterpret_cast<unsigned short*>(Vs + NST * VS_ELEMS);
     __shared__ int s_nblocks;
 
+    unsigned long long clk_c0 = 0, clk_r0 = 0;
+    if (a.clock_probe) {
+        clk_c0 = __builtin_readcyclecounter();
+        clk_r0 = __builtin_amdgcn_s_memrealtime();
+    }
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -633,6 +638,10 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                     }
             }
         }
+    }
+    if (a.clock_probe && tid == 0 && (int64_t)blockIdx.x < a.clock_cap) {
+        a.clock_probe[2 * blockIdx.x] = __builtin_readcyclecounter() - clk_c0;
+        a.clock_probe[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - clk_r0;
     }
 }
 

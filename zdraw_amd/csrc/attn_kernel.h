@@ -63,6 +63,10 @@ struct AttnArgs {
     // key-padding mask, u8 [segment][tokens], nonzero = key excluded; may be null
     const unsigned char* key_pad;
     int64_t mask_bs;    // bytes between segments (0 = shared)
+    // clock probe (null = off): workgroup i stores its run time as shader-clock
+    // cycles at [2i] and as ticks of the fixed 100 MHz reference at [2i+1], i < clock_cap
+    unsigned long long* clock_probe;
+    int64_t clock_cap;
 };
 
 // Standalone norm + rope over rows of one operand (Q or K): the pre-pass for

@@ -70,6 +70,15 @@ std::vector<TracePair> g_trace_open;
 uint64_t g_trace_ns = 0;
 uint64_t g_trace_launches = 0;
 
+// Clock probe: per-workgroup run time of the last traced attention launch in
+// shader-clock cycles and in 100 MHz reference ticks (their ratio is the clock
+// the kernel actually ran at, which under load is set by the power limit).
+constexpr int64_t kClockCap = 4096;
+bool g_clock_on = false;
+unsigned long long* g_clock_buf = nullptr;
+int64_t g_clock_wgs = 0;
+hipStream_t g_clock_stream = nullptr;
+
 thread_local char g_err[512] = "";
 
 void set_err(const char* fmt, ...) {
@@ -319,10 +328,20 @@ int enqueue(const FusedPlan& plan, hipStream_t stream) {
         }
         g_dispatch++;
     }
+    AttnArgs args = plan.args;
+    if (g_clock_on) {
+        if (!g_clock_buf && hipMalloc(&g_clock_buf, sizeof(unsigned long long) * 2 * kClockCap) != hipSuccess) g_clock_buf = nullptr;
+        if (g_clock_buf) {
+            args.clock_probe = g_clock_buf;
+            args.clock_cap = kClockCap;
+            g_clock_wgs = (int64_t)args.nqb * args.heads * args.batch;
+            g_clock_stream = stream;
+        }
+    }
     TracePair tp{nullptr, nullptr};
     if (g_trace && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
         (void)hipEventRecord(tp.a, stream);
-    hipError_t e = launch_attention(plan.args, plan.in_dtype, plan.k_mode, g_variant, stream);
+    hipError_t e = launch_attention(args, plan.in_dtype, plan.k_mode, g_variant, stream);
     if (e != hipSuccess) {
         set_err("attention launch: %s", hipGetErrorString(e));
         return ZDRAW_HIP_ERR_HANDLE;
@@ -763,6 +782,22 @@ uint64_t zdraw_hip_trace_attention_ns(uint64_t* launches) {
     g_trace_open.clear();
     if (launches) *launches = g_trace_launches;
     return g_trace_ns;
+}
+
+void zdraw_hip_clock_probe(int on) { g_clock_on = on != 0; }
+
+size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t capacity) {
+    if (!g_clock_buf || g_clock_wgs <= 0) return 0;
+    if (hipStreamSynchronize(g_clock_stream) != hipSuccess) return 0;
+    const size_t n = (size_t)(g_clock_wgs < kClockCap ? g_clock_wgs : kClockCap);
+    std::vector<unsigned long long> host(2 * n);
+    if (hipMemcpy(host.data(), g_clock_buf, sizeof(unsigned long long) * 2 * n, hipMemcpyDeviceToHost) != hipSuccess) return 0;
+    const size_t m = n < capacity ? n : capacity;
+    for (size_t i = 0; i < m; i++) {
+        if (cycles) cycles[i] = host[2 * i];
+        if (ref_ticks) ref_ticks[i] = host[2 * i + 1];
+    }
+    return m;
 }
 
 void zdraw_hip_set_attention_variant(int variant) { g_variant = variant == 1 ? 1 : 0; }

@@ -9,38 +9,38 @@
 namespace zdraw {
 
 // ------------------------------------------------ Q/K pre-pass (norm + rope)
-// 16 lanes per row (8 dims each). A workgroup covers 8 tokens x G heads of one
-// segment: a lane keeps the rope coefficients and norm weights of its token
-// and its 8 dims in registers and walks the G heads with them, so the rope
-// table is read once per token and head group, not once per row. All G loads
-// of a lane are issued before the first is used. Input and output are
+// 16 lanes per row (8 dims each). A wave covers one token: its four 16-lane
+// groups take four heads at a time (1 KB contiguous in a token-major operand)
+// and walk G such groups of heads, keeping the token's rope coefficients and
+// norm weights in registers, so the rope table is read once per token. All G
+// loads of a lane are issued before the first is used. Input and output are
 // addressed by strides, so the same kernel serves the bf16 K pre-pass and the
 // in-place f32 token-major form. A lane reads and writes only its own 8
 // elements, so the output may alias the input.
-constexpr int kPrepTokens = 8; // tokens per workgroup
-constexpr int kPrepHeads = 8;  // heads walked by one lane
+constexpr int kPrepTokens = 4; // tokens (waves) per workgroup
+constexpr int kPrepGroups = 6; // groups of four heads walked by one lane
 
 template <typename TIn>
-__global__ void __launch_bounds__(kPrepTokens * 16) qk_prepass_kernel(const PrepArgs p) {
-    constexpr int G = kPrepHeads;
-    const int tok_raw = (int)blockIdx.x * kPrepTokens + (int)(threadIdx.x >> 4);
+__global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const PrepArgs p) {
+    constexpr int G = kPrepGroups;
+    const int tok_raw = (int)blockIdx.x * kPrepTokens + (int)(threadIdx.x >> 6);
     const bool tok_ok = tok_raw < p.tokens;
     const int tok = tok_ok ? tok_raw : 0;
-    const int h0 = (int)blockIdx.y * G;
+    const int h0 = (int)blockIdx.y * (4 * G) + (int)((threadIdx.x >> 4) & 3);
     const int seg = (int)blockIdx.z;
     const int d0 = (threadIdx.x & 15) * 8;
     const TIn* src = reinterpret_cast<const TIn*>(p.x) + (int64_t)seg * p.x_bs + (int64_t)tok * p.x_ts + d0;
     Raw8<TIn> raw[G];
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        const int head = h0 + g;
+        const int head = h0 + 4 * g;
         raw[g] = ld_raw8<TIn>(src + (int64_t)(head < p.heads ? head : 0) * p.x_hs, tok_ok && head < p.heads);
     }
     const QkRow qr = qk_row(p.qk, p.mode, p.w, p.w_txt, seg, tok, tok_ok);
     const Rope8 t = ld_rope8(p.qk, p.mode, qr, d0);
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        const int head = h0 + g;
+        const int head = h0 + 4 * g;
         float x[8];
         unpack8(raw[g], x);
         float ss = 0.f;
@@ -64,9 +64,9 @@ __global__ void __launch_bounds__(kPrepTokens * 16) qk_prepass_kernel(const Prep
 
 hipError_t launch_qk_prepass(const PrepArgs& p, int in_dtype, hipStream_t stream) {
     if (p.batch <= 0 || p.heads <= 0 || p.tokens <= 0 || p.batch > 65535) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)((p.tokens + kPrepTokens - 1) / kPrepTokens), (unsigned)((p.heads + kPrepHeads - 1) / kPrepHeads),
-                    (unsigned)p.batch);
-    const dim3 block(kPrepTokens * 16);
+    const dim3 grid((unsigned)((p.tokens + kPrepTokens - 1) / kPrepTokens),
+                    (unsigned)((p.heads + 4 * kPrepGroups - 1) / (4 * kPrepGroups)), (unsigned)p.batch);
+    const dim3 block(kPrepTokens * 64);
     if (in_dtype == kF32)
         qk_prepass_kernel<float><<<grid, block, 0, stream>>>(p);
     else if (in_dtype == kBF16)

@@ -76,6 +76,9 @@ SYMBOLS = {
     "zdraw_hip_gpu_ns": (_u64, []),
     "zdraw_hip_trace_attention": (None, [_int]),
     "zdraw_hip_trace_attention_ns": (_u64, [C.POINTER(C.c_uint64)]),
+    "zdraw_hip_mfma_probe": (_int, [_int, _int, C.POINTER(C.c_double)]),
+    "zdraw_hip_clock_probe": (None, [_int]),
+    "zdraw_hip_clock_probe_read": (C.c_size_t, [C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_size_t]),
     "zdraw_hip_event_create": (_vp, []),
     "zdraw_hip_event_record": (_int, [_vp, _vp]),
     "zdraw_hip_event_sync": (_int, [_vp]),
