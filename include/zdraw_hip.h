@@ -140,8 +140,8 @@ void zdraw_hip_release_buffer(void* buffer);
 
 /* ---- pipelines (metal_c.zig:99-107) -------------------------------------- */
 /* The kernels are compiled ahead of time for gfx950, so "compile" is a lookup
- * by entry name: "attention_block_mfma" (the only attention pipeline) and
- * "qk_norm_rope". Unknown names return NULL and write a message. */
+ * by entry name: "attention_block_mfma" (the only attention pipeline),
+ * "qk_norm_rope" and "gemm_half". Unknown names return NULL and write a message. */
 void* zdraw_hip_compile(void* device, const char* entry, char* error_buf, size_t error_len);
 void zdraw_hip_release_pipeline(void* pipeline);
 size_t zdraw_hip_pipeline_threads(void* pipeline);
@@ -181,6 +181,51 @@ int zdraw_hip_run_attention_fused(void* queue, void* q, void* k, void* v, void* 
 int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
                                const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
                                const ZdrawHipQkOperands* ops);
+
+/* ---- projections either side of attention: C = A x W^T ----------------------
+ * metal_c.zig:276-283 (GemmParams), same field order, 32 bytes. dtype is the
+ * WEIGHT's type in the reference's coding (metal/mres_util.zig:11-18): 1 = f16,
+ * 2 = bf16, 3 = f32; mode is metal/mgemm.zig:225-233: 2 = half (operands
+ * rounded to the weight's 16-bit type, fp32 accumulation), 1 = exact f32.
+ * This backend computes mode 2 with 16-bit weights; everything else (exact
+ * mode, f32 or packed W8/W6/W4 weights, k % 8 != 0) returns 1 = unavailable
+ * and the caller keeps its own path (runtime/linear_fast.zig:14-29). */
+typedef struct ZdrawGemmParams {
+    uint32_t m;  /* rows of A and C */
+    uint32_t k;  /* columns of A and of W */
+    uint32_t n;  /* rows of W, columns of C */
+    uint32_t dtype;
+    uint32_t mode;
+    uint64_t weight_offset; /* byte offset of W in its buffer */
+} ZdrawGemmParams;
+enum { ZDRAW_HIP_W_F16 = 1, ZDRAW_HIP_W_BF16 = 2, ZDRAW_HIP_W_F32 = 3 };
+enum { ZDRAW_HIP_GEMM_EXACT = 1, ZDRAW_HIP_GEMM_HALF = 2 };
+
+/* What the reference passes as byte offsets only, plus leading dimensions and
+ * 16-bit activations / outputs (no counterpart struct in the reference).
+ * Leading dimensions are in elements; 0 means dense (k, k, n). */
+typedef struct ZdrawHipGemmExt {
+    uint64_t a_off, c_off; /* byte offsets into the A and C buffers */
+    uint64_t lda, ldw, ldc;
+    uint32_t a_dtype;      /* ZDRAW_HIP_F32, or the weight's type (ZDRAW_HIP_F16 / ZDRAW_HIP_BF16) */
+    uint32_t c_dtype;      /* ZDRAW_HIP_F32, or the weight's type */
+} ZdrawHipGemmExt;
+
+/* metal_c.zig:160-167: A f32 [m][k], W [n][k], C f32 [m][n]; blocks until done.
+ * pipeline is zdraw_hip_compile(device, "gemm_half", ...). */
+int zdraw_hip_run_gemm(void* queue, void* pipeline, void* a, void* w, void* c, const ZdrawGemmParams* params);
+/* metal_c.zig:357-364, 368-377: the same inside a batch, and with A / C byte offsets. */
+int zdraw_hip_run_gemm_enc(void* batch, void* pipeline, void* a, void* w, void* c, const ZdrawGemmParams* params);
+int zdraw_hip_run_gemm_off_enc(void* batch, void* pipeline, void* a, void* w, void* c,
+                               const ZdrawGemmParams* params, uint64_t a_offset, uint64_t c_offset);
+/* metal_c.zig:425-433 (and :378-386): A already in the weight's 16-bit type, C f32. */
+int zdraw_hip_run_gemm_f16a_enc(void* batch, void* a, void* w, void* c, const ZdrawGemmParams* params,
+                                uint64_t a_offset, uint64_t c_offset);
+/* General form: leading dimensions and 16-bit output, e.g. Q/K/V written as
+ * bf16 token-major rows for the attention entry, or the attention output read
+ * from the concat operand at its row pitch. */
+int zdraw_hip_run_gemm_ext_enc(void* batch, void* a, void* w, void* c, const ZdrawGemmParams* params,
+                               const ZdrawHipGemmExt* ext);
 
 /* ---- library-owned scratch (metal_c.zig:321-325) -------------------------- */
 /* Grow-only, process-lifetime, filled at (re)allocation with 0x00 (0xFF when
@@ -233,7 +278,8 @@ void zdraw_hip_set_attention_variant(int variant);
 
 /* ABI drift guard (src/abi_gen.zig, runtime/abi_assert.zig:29): sizeof of the
  * shared structs as this library was compiled. which: 0 = ZdrawAttnParams,
- * 1 = ZdrawHipAttnExt, 2 = ZdrawHipQkOperands. */
+ * 1 = ZdrawHipAttnExt, 2 = ZdrawHipQkOperands, 3 = ZdrawGemmParams,
+ * 4 = ZdrawHipGemmExt. */
 size_t zdraw_hip_abi_sizeof(int which);
 /* Last error text of this thread's most recent failing call ("" if none). */
 const char* zdraw_hip_last_error(void);
@@ -241,6 +287,8 @@ const char* zdraw_hip_last_error(void);
 #define ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE 24
 #define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 216
 #define ZDRAW_HIP_ABI_QK_OPERANDS_SIZE 72
+#define ZDRAW_HIP_ABI_GEMM_PARAMS_SIZE 32
+#define ZDRAW_HIP_ABI_GEMM_EXT_SIZE 48
 
 #ifdef __cplusplus
 }

@@ -32,6 +32,9 @@
  *   zo_zseq_*, zo_zunify_basic    pinned: zseq.zig:94-133, zunify.zig:47-66.
  *   zo_read_f32 (f16/bf16 decode) pinned: ops.zig:137-174 byte vectors and
  *                                 numpy's float16 / bit-shifted bf16 decode.
+ *   zo_linear_batch               pinned: mlinear_test.zig:33-80 known answers,
+ *                                 the bf16 case of mlinear_test.zig:82-121,
+ *                                 numpy float64 matmul, linearity.
  */
 #ifndef ZDRAW_ORACLE_H
 #define ZDRAW_ORACLE_H
@@ -148,6 +151,12 @@ int zo_zunify_basic(float* out, size_t out_len, size_t* pos_out, size_t pos_out_
 
 /* pack/tensor.zig:108-147 (readF32 / fromBits): dtype 0=f32, 1=f16, 2=bf16, 3=u8. */
 float zo_read_f32(int dtype, const uint8_t* bytes);
+
+/* ---- dense projection (runtime/ops.zig:37-60, metal/mgemm.zig:134-155) -------
+ * out [count][rows] = input [count][cols] x weight[rows][cols]^T (+ bias[rows]),
+ * fp32, columns accumulated in order. bias may be NULL. */
+int zo_linear_batch(float *out, size_t out_len, const float *input, size_t input_len, const float *weight,
+                    size_t weight_len, const float *bias, size_t rows, size_t cols, size_t count);
 
 #ifdef __cplusplus
 }

@@ -20,6 +20,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libzdraw_oracle.so")
 
 OK, INVALID_SHAPE, INVALID_CONFIG, BAD_POSITION = 0, 1, 2, 3
+DT_F32, DT_F16, DT_BF16 = 0, 1, 2  # dtype codes of read_f32 (pack/tensor.zig:108-115)
 
 
 class OracleError(Exception):
@@ -136,6 +137,9 @@ def lib():
                                       C.c_size_t, _fp, C.c_size_t, _sp, C.c_size_t, C.c_size_t]
         L.zo_read_f32.restype = C.c_float
         L.zo_read_f32.argtypes = [C.c_int, _bp]
+        L.zo_linear_batch.restype = C.c_int
+        L.zo_linear_batch.argtypes = [_fp, C.c_size_t, _fp, C.c_size_t, _fp, C.c_size_t, _fp,
+                                      C.c_size_t, C.c_size_t, C.c_size_t]
         _lib = L
     return _lib
 
@@ -337,3 +341,18 @@ def zunify_basic(image, image_pos, cap, cap_pos, hidden):
 def read_f32(dtype: int, raw: bytes) -> float:
     buf = (C.c_uint8 * 4)(*(list(raw) + [0] * (4 - len(raw))))
     return float(lib().zo_read_f32(dtype, buf))
+
+
+def linear_batch(x, weight, bias=None) -> np.ndarray:
+    """runtime/ops.zig:37-60 over rows (metal/mgemm.zig:134-155): x [count][cols], weight [rows][cols]
+    already decoded to fp32 -> [count][rows]."""
+    x, weight = f32(x), f32(weight)
+    if x.ndim != 2 or weight.ndim != 2:
+        raise OracleError(INVALID_SHAPE)
+    count, cols = x.shape
+    rows = weight.shape[0]
+    out = np.empty((count, rows), np.float32)
+    b = f32(bias) if bias is not None else None
+    _check(lib().zo_linear_batch(_f(out), out.size, _f(x), x.size, _f(weight), weight.size,
+                                 _f(b) if b is not None else None, rows, weight.shape[1] if x.size else cols, count))
+    return out

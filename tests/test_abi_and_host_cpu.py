@@ -36,10 +36,16 @@ def test_abi_struct_sizes():
     assert L.zdraw_hip_abi_sizeof(0) == 24 == C.sizeof(hip.AttnParams)
     assert L.zdraw_hip_abi_sizeof(1) == C.sizeof(hip.AttnExt) == 216
     assert L.zdraw_hip_abi_sizeof(2) == C.sizeof(hip.QkOperands) == 72
+    # GemmParams keeps the reference's 32-byte layout (metal_c.zig:276-283)
+    assert L.zdraw_hip_abi_sizeof(3) == C.sizeof(hip.GemmParams) == 32
+    assert hip.GemmParams.weight_offset.offset == 24
+    assert L.zdraw_hip_abi_sizeof(4) == C.sizeof(hip.GemmExt) == 48
     text = open(os.path.join(ROOT, "include", "zdraw_hip.h")).read()
     assert "#define ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE 24" in text
     assert "#define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 216" in text
     assert "#define ZDRAW_HIP_ABI_QK_OPERANDS_SIZE 72" in text
+    assert "#define ZDRAW_HIP_ABI_GEMM_PARAMS_SIZE 32" in text
+    assert "#define ZDRAW_HIP_ABI_GEMM_EXT_SIZE 48" in text
 
 
 def test_pipeline_lookup_without_device_is_null():

@@ -1,0 +1,201 @@
+"""Parity of the projection GEMM (C = A x W^T) with the CPU oracle, through the
+C ABI. The reference's half mode rounds both operands to the weight's 16-bit
+type and accumulates in fp32 (metal/mgemm.zig, gemm_mode.zig); so does the
+kernel. Two bars, both stated where they are used:
+  * against the oracle fed the SAME rounded operands only the summation order
+    differs: |err| <= 2e-5 * sqrt(k) * (rms of A) * (rms of W) ... in practice 1e-6 relative;
+  * against the fp32 oracle on the un-rounded operands: max |err| <= 2e-2 * s,
+    mean |err| <= 2e-3 * s with s = sqrt(k) * rms(A) * rms(W) (the attention
+    path's tolerance in units of the output's scale).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import zoracle as zo
+from zdraw_amd import hip, host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = host.Context.init()
+    yield c
+    c.deinit()
+
+
+@pytest.fixture(scope="module")
+def pipe(ctx):
+    L = hip.lib()
+    err = C.create_string_buffer(128)
+    p = L.zdraw_hip_compile(ctx.device, b"gemm_half", err, 128)
+    assert p, err.value
+    yield p
+    L.zdraw_hip_release_pipeline(p)
+
+
+def to16(x, wdt):
+    """fp32 -> the 16-bit type's bits and the value they decode to."""
+    if wdt == hip.W_BF16:
+        bits = host.f32_to_bf16_bits(x)
+        return bits, host.bf16_bits_to_f32(bits)
+    h = x.astype(np.float16)
+    return h.view(np.uint16), h.astype(np.float32)
+
+
+def from16(bits, wdt):
+    return host.bf16_bits_to_f32(bits) if wdt == hip.W_BF16 else bits.view(np.float16).astype(np.float32)
+
+
+def act_dtype(wdt):
+    return hip.BF16 if wdt == hip.W_BF16 else hip.F16
+
+
+def run_ext(ctx, a_host, w_bits, m, k, n, wdt, a_dtype, c_dtype, lda=0, ldc=0, a_off=0, c_off=0, c_init=None):
+    L = hip.lib()
+    ab, wb = ctx.buffer(a_host), ctx.buffer(w_bits)
+    esz = 4 if c_dtype == hip.F32 else 2
+    rows = m
+    pitch = ldc or n
+    cb = ctx.buffer(c_init) if c_init is not None else ctx.buffer(nbytes=c_off + rows * pitch * esz)
+    params = hip.GemmParams(m, k, n, wdt, hip.GEMM_HALF, 0)
+    ext = hip.GemmExt(a_off, c_off, lda, 0, ldc, a_dtype, c_dtype)
+    batch = L.zdraw_hip_batch_begin(ctx.queue)
+    rc = L.zdraw_hip_run_gemm_ext_enc(batch, ab.handle, wb.handle, cb.handle, C.byref(params), C.byref(ext))
+    assert L.zdraw_hip_batch_end(batch) == 0
+    assert rc == 0, hip.last_error()
+    raw = cb.read(np.uint8, (cb.nbytes,))
+    for b in (ab, wb, cb):
+        b.release()
+    return raw
+
+
+def check(got, want_same_rounding, want_fp32, k, a, w, what):
+    s = np.sqrt(k) * np.sqrt(np.mean(a.astype(np.float64) ** 2)) * np.sqrt(np.mean(w.astype(np.float64) ** 2))
+    e1 = np.abs(got - want_same_rounding)
+    assert e1.max() <= 2e-5 * s + 1e-6, f"{what}: vs oracle on rounded operands max {e1.max():.3e} (scale {s:.3e})"
+    e2 = np.abs(got - want_fp32)
+    assert e2.max() <= 2e-2 * s and e2.mean() <= 2e-3 * s, f"{what}: vs fp32 oracle max {e2.max():.3e} mean {e2.mean():.3e}"
+
+
+def test_reference_bf16_ffn_shaped_case(ctx, pipe):
+    # mlinear_test.zig:82-121 through the blocking entry (metal_c.zig:160-167): f32 A, bf16 W, f32 C, tolerance 0.005
+    L = hip.lib()
+    m, k, n = 32, 8, 32
+    x = ((np.arange(m * k) % 7).astype(np.float32) * np.float32(0.1) - np.float32(0.3)).reshape(m, k)
+    raw = (np.arange(n * k) % 11).astype(np.float32) * np.float32(0.05) - np.float32(0.25)
+    hi = (raw.view(np.uint32) >> 16).astype(np.uint16).reshape(n, k)
+    wv = host.bf16_bits_to_f32(hi)
+    ab, wb, cb = ctx.buffer(x), ctx.buffer(hi), ctx.buffer(nbytes=m * n * 4)
+    params = hip.GemmParams(m, k, n, hip.W_BF16, hip.GEMM_HALF, 0)
+    assert L.zdraw_hip_run_gemm(ctx.queue, pipe, ab.handle, wb.handle, cb.handle, C.byref(params)) == 0, hip.last_error()
+    got = cb.read(np.float32, (m, n))
+    want = zo.linear_batch(x, wv)
+    assert np.abs(got - want).max() <= 0.005
+    for b in (ab, wb, cb):
+        b.release()
+
+
+def test_small_known_answer_shapes_take_the_fallback_contract(ctx, pipe):
+    # mlinear_test.zig:33-46 is 2 x 2: below this backend's k % 8 granule -> 1 = unavailable,
+    # nothing enqueued, the caller keeps its own path (runtime/linear_fast.zig:14-29)
+    L = hip.lib()
+    ab, wb, cb = ctx.buffer(np.zeros(16, np.float32)), ctx.buffer(np.zeros(16, np.uint16)), ctx.buffer(nbytes=64)
+    d0, f0 = L.zdraw_hip_dispatch_count(), L.zdraw_hip_attn_fallback_count()
+    for params in (hip.GemmParams(1, 2, 2, hip.W_F16, hip.GEMM_HALF, 0),      # k % 8 != 0
+                   hip.GemmParams(8, 8, 8, hip.W_F32, hip.GEMM_HALF, 0),      # f32 weights
+                   hip.GemmParams(8, 8, 8, hip.W_BF16, hip.GEMM_EXACT, 0),    # exact mode
+                   hip.GemmParams(8, 8, 8, 4, 4, 0)):                         # packed W6
+        assert L.zdraw_hip_run_gemm(ctx.queue, pipe, ab.handle, wb.handle, cb.handle, C.byref(params)) == 1
+    assert L.zdraw_hip_dispatch_count() == d0 and L.zdraw_hip_attn_fallback_count() == f0 + 4
+    # malformed: buffer too small, zero dimension
+    assert L.zdraw_hip_run_gemm(ctx.queue, pipe, ab.handle, wb.handle, cb.handle,
+                                C.byref(hip.GemmParams(64, 64, 64, hip.W_BF16, hip.GEMM_HALF, 0))) == 2
+    assert L.zdraw_hip_run_gemm(ctx.queue, pipe, ab.handle, wb.handle, cb.handle,
+                                C.byref(hip.GemmParams(0, 8, 8, hip.W_BF16, hip.GEMM_HALF, 0))) == 2
+    for b in (ab, wb, cb):
+        b.release()
+
+
+SHAPES = [(32, 64, 32), (256, 64, 256), (300, 72, 260), (513, 200, 257), (64, 1024, 96), (600, 320, 520)]
+
+
+@pytest.mark.parametrize("wdt", [hip.W_BF16, hip.W_F16])
+@pytest.mark.parametrize("a16", [False, True])
+@pytest.mark.parametrize("c16", [False, True])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_random_matrices_against_the_oracle(ctx, shape, wdt, a16, c16):
+    m, k, n = shape
+    rng = np.random.default_rng(m * 7 + k * 3 + n)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.5)
+    w_bits, w_val = to16(w, wdt)
+    a_bits, a_val = to16(a, wdt)
+    adt = act_dtype(wdt)
+    raw = run_ext(ctx, a_bits if a16 else a, w_bits, m, k, n, wdt, adt if a16 else hip.F32, adt if c16 else hip.F32)
+    got = from16(raw.view(np.uint16).reshape(m, n), wdt) if c16 else raw.view(np.float32).reshape(m, n)
+    same = zo.linear_batch(a_val, w_val)          # the kernel rounds f32 activations exactly like to16()
+    full = zo.linear_batch(a, w)
+    if c16:  # the output rounding adds half an ulp of the 16-bit type
+        same = from16(to16(same, wdt)[0], wdt)
+        s = np.sqrt(k) * a.std() * w.std()
+        assert np.abs(got - same).max() <= (2.0 ** -7 if wdt == hip.W_BF16 else 2.0 ** -10) * np.abs(same).max() + 2e-5 * s
+        e2 = np.abs(got - full)
+        assert e2.max() <= 3e-2 * s and e2.mean() <= 4e-3 * s
+    else:
+        check(got, same, full, k, a, w, f"{shape} wdt={wdt} a16={a16}")
+
+
+def test_offsets_and_leading_dimensions(ctx):
+    # a stream's rows written straight into a shared, wider C at a row/column offset
+    # (klein/zflux2_resident.zig:1467-1513), A read from a wider matrix
+    m, k, n = 70, 96, 40
+    lda, ldc = 128, 200
+    rng = np.random.default_rng(3)
+    big_a = rng.standard_normal((m + 5, lda), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32)
+    w_bits, w_val = to16(w, hip.W_BF16)
+    a_row0, a_col0, c_row0, c_col0 = 3, 16, 9, 24
+    c_rows = c_row0 + m + 2
+    c_init = np.full((c_rows, ldc), 7.0, np.float32)
+    raw = run_ext(ctx, big_a, w_bits, m, k, n, hip.W_BF16, hip.F32, hip.F32, lda=lda, ldc=ldc,
+                  a_off=(a_row0 * lda + a_col0) * 4, c_off=(c_row0 * ldc + c_col0) * 4, c_init=c_init)
+    got = raw.view(np.float32).reshape(c_rows, ldc)
+    a = np.ascontiguousarray(big_a[a_row0:a_row0 + m, a_col0:a_col0 + k])
+    want = zo.linear_batch(host.bf16_bits_to_f32(host.f32_to_bf16_bits(a)), w_val)
+    block = got[c_row0:c_row0 + m, c_col0:c_col0 + n]
+    check(block, want, zo.linear_batch(a, w), k, a, w, "offset block")
+    mask = np.ones_like(got, bool)
+    mask[c_row0:c_row0 + m, c_col0:c_col0 + n] = False
+    assert (got[mask] == 7.0).all(), "wrote outside the addressed block"
+
+
+def test_reference_offset_entries_and_bit_stability(ctx, pipe):
+    # zdraw_metal_run_gemm_off_enc / _f16a_enc: f32 (or 16-bit) A at a byte offset, f32 C at a byte offset
+    L = hip.lib()
+    m, k, n = 96, 128, 64
+    rng = np.random.default_rng(9)
+    a = rng.standard_normal((2 * m, k), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32)
+    w_bits, w_val = to16(w, hip.W_F16)
+    a_bits, a_val = to16(a, hip.W_F16)
+    ab, a16b, wb = ctx.buffer(a), ctx.buffer(a_bits), ctx.buffer(w_bits)
+    cb = ctx.buffer(nbytes=2 * m * n * 4)
+    params = hip.GemmParams(m, k, n, hip.W_F16, hip.GEMM_HALF, 0)
+    outs = []
+    for rep in range(3):
+        batch = L.zdraw_hip_batch_begin(ctx.queue)
+        assert L.zdraw_hip_run_gemm_off_enc(batch, pipe, ab.handle, wb.handle, cb.handle, C.byref(params),
+                                            m * k * 4, m * n * 4) == 0, hip.last_error()
+        assert L.zdraw_hip_run_gemm_f16a_enc(batch, a16b.handle, wb.handle, cb.handle, C.byref(params), 0, 0) == 0
+        assert L.zdraw_hip_batch_end(batch) == 0
+        outs.append(cb.read(np.float32, (2, m, n)))
+    assert all(np.array_equal(outs[0].view(np.uint32), o.view(np.uint32)) for o in outs[1:])
+    want = zo.linear_batch(a_val, w_val).reshape(2, m, n)
+    s = np.sqrt(k) * a.std() * w.std()
+    assert np.abs(outs[0][1] - want[1]).max() <= 2e-5 * s   # off_enc: second half of A -> second half of C
+    assert np.abs(outs[0][0] - want[0]).max() <= 2e-5 * s   # f16a_enc: first half, A already half
+    for b in (ab, a16b, wb, cb):
+        b.release()

@@ -9,6 +9,7 @@
 // take the whole device down.
 #include "../../include/zdraw_hip.h"
 #include "attn_kernel.h"
+#include "gemm_kernel.h"
 
 #include <hip/hip_runtime.h>
 
@@ -24,6 +25,8 @@ using namespace zdraw;
 static_assert(sizeof(ZdrawAttnParams) == ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE, "AttnParams ABI drift");
 static_assert(sizeof(ZdrawHipAttnExt) == ZDRAW_HIP_ABI_ATTN_EXT_SIZE, "AttnExt ABI drift");
 static_assert(sizeof(ZdrawHipQkOperands) == ZDRAW_HIP_ABI_QK_OPERANDS_SIZE, "QkOperands ABI drift");
+static_assert(sizeof(ZdrawGemmParams) == ZDRAW_HIP_ABI_GEMM_PARAMS_SIZE, "GemmParams ABI drift");
+static_assert(sizeof(ZdrawHipGemmExt) == ZDRAW_HIP_ABI_GEMM_EXT_SIZE, "GemmExt ABI drift");
 
 namespace {
 
@@ -40,7 +43,7 @@ struct Buffer {
     bool owned;
 };
 struct Pipeline {
-    int kind; // 0 = attention_block_mfma, 1 = qk_norm_rope
+    int kind; // 0 = attention_block_mfma, 1 = qk_norm_rope, 2 = gemm_half
 };
 struct Batch {
     Queue* queue;
@@ -58,6 +61,7 @@ uint64_t g_fallback = 0;
 uint64_t g_gpu_ns = 0;
 int g_variant = 0; // kernel shape: 0 = 8 waves per workgroup, 1 = 4 waves (two workgroups per CU)
 bool g_setup_done = false;
+bool g_gemm_setup_done = false;
 
 // Attention-kernel trace (the reference's ZDRAW_KLEIN_TRACE attention bucket,
 // klein/zflux2_resident.zig:443-467): when on, every attention launch is
@@ -410,6 +414,65 @@ bool scratch_poisoned(int slot) {
     return false;
 }
 
+// C = A x W^T (metal_api.m gemm encode paths). Validates, then launches on `stream`.
+int enqueue_gemm(void* a, void* w, void* c, const ZdrawGemmParams* p, const ZdrawHipGemmExt* x, hipStream_t stream) {
+    if (!p || !x) {
+        set_err("null params");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    if (p->m == 0 || p->k == 0 || p->n == 0) return invalid("zero dimension");
+    if (p->mode != ZDRAW_HIP_GEMM_HALF) return unavailable("only the half-precision GEMM mode exists");
+    if (p->dtype != ZDRAW_HIP_W_F16 && p->dtype != ZDRAW_HIP_W_BF16) return unavailable("weight dtype");
+    if (p->k % 8 != 0) return unavailable("k % 8 != 0");
+    const uint32_t wt = p->dtype == ZDRAW_HIP_W_F16 ? (uint32_t)ZDRAW_HIP_F16 : (uint32_t)ZDRAW_HIP_BF16;
+    if ((x->a_dtype != ZDRAW_HIP_F32 && x->a_dtype != wt) || (x->c_dtype != ZDRAW_HIP_F32 && x->c_dtype != wt))
+        return invalid("activation / output dtype must be f32 or the weight's type");
+    const Buffer* ab = static_cast<const Buffer*>(a);
+    const Buffer* wb = static_cast<const Buffer*>(w);
+    const Buffer* cb = static_cast<const Buffer*>(c);
+    if (!ab || !wb || !cb || !ab->ptr || !wb->ptr || !cb->ptr) return invalid("null buffer");
+    const uint64_t lda = x->lda ? x->lda : p->k, ldw = x->ldw ? x->ldw : p->k, ldc = x->ldc ? x->ldc : p->n;
+    if (lda < p->k || ldw < p->k || ldc < p->n) return invalid("leading dimension smaller than the row");
+    const uint64_t ea = elem_size(x->a_dtype), ec = elem_size(x->c_dtype);
+    // 16-byte loads of 8 (16-bit) or 4 (f32) elements: rows must start 16-byte aligned
+    if (x->a_off % 16 != 0 || (lda * ea) % 16 != 0 || ((uintptr_t)ab->ptr % 16) != 0) return invalid("A rows not 16-byte aligned");
+    if (p->weight_offset % 16 != 0 || (ldw * 2) % 16 != 0 || ((uintptr_t)wb->ptr % 16) != 0) return invalid("W rows not 16-byte aligned");
+    if (x->c_off % ec != 0) return invalid("C offset not element aligned");
+    const uint64_t a_bytes = ((uint64_t)(p->m - 1) * lda + p->k) * ea;
+    const uint64_t w_bytes = ((uint64_t)(p->n - 1) * ldw + p->k) * 2;
+    const uint64_t c_bytes = ((uint64_t)(p->m - 1) * ldc + p->n) * ec;
+    if (x->a_off > ab->len || a_bytes > ab->len - x->a_off) return invalid("A buffer too small");
+    if (p->weight_offset > wb->len || w_bytes > wb->len - p->weight_offset) return invalid("W buffer too small");
+    if (x->c_off > cb->len || c_bytes > cb->len - x->c_off) return invalid("C buffer too small");
+    // the kernel addresses A and W with 32-bit byte offsets from their first element
+    if (a_bytes >= (1ull << 32) || w_bytes >= (1ull << 32)) return unavailable("operand spans 4 GiB or more");
+    if (!g_gemm_setup_done) {
+        hipError_t e = gemm_setup();
+        if (e != hipSuccess) {
+            set_err("gemm_setup: %s", hipGetErrorString(e));
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        g_gemm_setup_done = true;
+    }
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.a = static_cast<const char*>(ab->ptr) + x->a_off;
+    g.w = static_cast<const char*>(wb->ptr) + p->weight_offset;
+    g.c = static_cast<char*>(cb->ptr) + x->c_off;
+    g.m = (int32_t)p->m; g.n = (int32_t)p->n; g.k = (int32_t)p->k;
+    g.lda = (int64_t)lda; g.ldw = (int64_t)ldw; g.ldc = (int64_t)ldc;
+    g.tiles_n = (int32_t)((p->n + (uint32_t)gemm_tile_cols() - 1) / (uint32_t)gemm_tile_cols());
+    if ((uint64_t)g.tiles_n * ((p->m + (uint32_t)gemm_tile_rows() - 1) / (uint32_t)gemm_tile_rows()) > 0x7fffffffull)
+        return unavailable("grid too large");
+    hipError_t e = launch_gemm(g, (int)x->a_dtype, (int)wt, (int)x->c_dtype, stream);
+    if (e != hipSuccess) {
+        set_err("gemm launch: %s", hipGetErrorString(e));
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    g_dispatch++;
+    return ZDRAW_HIP_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -521,6 +584,7 @@ void* zdraw_hip_compile(void* device, const char* entry, char* error_buf, size_t
     if (!device || !entry) return nullptr;
     if (strcmp(entry, "attention_block_mfma") == 0) return new Pipeline{0};
     if (strcmp(entry, "qk_norm_rope") == 0) return new Pipeline{1};
+    if (strcmp(entry, "gemm_half") == 0) return new Pipeline{2};
     if (error_buf && error_len) snprintf(error_buf, error_len, "no gfx950 kernel named '%s'", entry);
     return nullptr;
 }
@@ -530,6 +594,7 @@ void zdraw_hip_release_pipeline(void* pipeline) { delete static_cast<Pipeline*>(
 size_t zdraw_hip_pipeline_threads(void* pipeline) {
     Pipeline* p = static_cast<Pipeline*>(pipeline);
     if (!p) return 0;
+    if (p->kind == 2) return 512;
     return p->kind == 0 ? (g_variant == 0 ? 512 : 256) : 256;
 }
 
@@ -692,6 +757,60 @@ int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
     return ZDRAW_HIP_OK;
 }
 
+// --------------------------------------------------------------------- gemm
+int zdraw_hip_run_gemm_ext_enc(void* batch, void* a, void* w, void* c, const ZdrawGemmParams* params,
+                               const ZdrawHipGemmExt* ext) {
+    Batch* b = static_cast<Batch*>(batch);
+    if (!b) {
+        set_err("null batch");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    return enqueue_gemm(a, w, c, params, ext, b->queue->stream);
+}
+
+int zdraw_hip_run_gemm_off_enc(void* batch, void* pipeline, void* a, void* w, void* c,
+                               const ZdrawGemmParams* params, uint64_t a_offset, uint64_t c_offset) {
+    int rc = check_pipeline(pipeline, 0, 2);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    ZdrawHipGemmExt x;
+    memset(&x, 0, sizeof(x));
+    x.a_off = a_offset;
+    x.c_off = c_offset;
+    x.a_dtype = ZDRAW_HIP_F32;
+    x.c_dtype = ZDRAW_HIP_F32;
+    return zdraw_hip_run_gemm_ext_enc(batch, a, w, c, params, &x);
+}
+
+int zdraw_hip_run_gemm_enc(void* batch, void* pipeline, void* a, void* w, void* c, const ZdrawGemmParams* params) {
+    return zdraw_hip_run_gemm_off_enc(batch, pipeline, a, w, c, params, 0, 0);
+}
+
+int zdraw_hip_run_gemm_f16a_enc(void* batch, void* a, void* w, void* c, const ZdrawGemmParams* params,
+                                uint64_t a_offset, uint64_t c_offset) {
+    if (!params) {
+        set_err("null params");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    ZdrawHipGemmExt x;
+    memset(&x, 0, sizeof(x));
+    x.a_off = a_offset;
+    x.c_off = c_offset;
+    x.a_dtype = params->dtype == ZDRAW_HIP_W_F16 ? ZDRAW_HIP_F16 : ZDRAW_HIP_BF16;
+    x.c_dtype = ZDRAW_HIP_F32;
+    return zdraw_hip_run_gemm_ext_enc(batch, a, w, c, params, &x);
+}
+
+int zdraw_hip_run_gemm(void* queue, void* pipeline, void* a, void* w, void* c, const ZdrawGemmParams* params) {
+    void* b = zdraw_hip_batch_begin(queue);
+    if (!b) {
+        set_err("null queue");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    int rc = zdraw_hip_run_gemm_enc(b, pipeline, a, w, c, params);
+    int rc2 = zdraw_hip_batch_end(b);
+    return rc != ZDRAW_HIP_OK ? rc : rc2;
+}
+
 // ------------------------------------------------------------------ scratch
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes) {
     if (!device || slot < 0 || slot >= 5 || bytes == 0) return nullptr;
@@ -807,6 +926,8 @@ size_t zdraw_hip_abi_sizeof(int which) {
     case 0: return sizeof(ZdrawAttnParams);
     case 1: return sizeof(ZdrawHipAttnExt);
     case 2: return sizeof(ZdrawHipQkOperands);
+    case 3: return sizeof(ZdrawGemmParams);
+    case 4: return sizeof(ZdrawHipGemmExt);
     default: return 0;
     }
 }

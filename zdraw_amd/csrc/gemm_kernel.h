@@ -1,0 +1,28 @@
+// Internal interface of the 16-bit MFMA GEMM that feeds and drains attention.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace zdraw {
+
+// C[m][n] = A[m][k] x W[n][k]^T, fp32 accumulation, operands rounded to the
+// weight's 16-bit type. Leading dimensions are in elements.
+struct GemmArgs {
+    const void* a;   // activations, row-major [m][lda]
+    const void* w;   // weights, row-major [n][ldw]
+    void* c;         // output, row-major [m][ldc]
+    int32_t m, n, k;
+    int32_t pad0;
+    int64_t lda, ldw, ldc;
+    int32_t tiles_n; // column tiles (grid = tiles_m * tiles_n)
+    int32_t pad1;
+};
+
+int gemm_tile_rows();
+int gemm_tile_cols();
+// a_dtype: kF32 or the weight's type; w_dtype: kF16 or kBF16; c_dtype: kF32 or the weight's type.
+hipError_t launch_gemm(const GemmArgs& args, int a_dtype, int w_dtype, int c_dtype, hipStream_t stream);
+hipError_t gemm_setup();
+
+} // namespace zdraw

@@ -41,9 +41,25 @@ class QkOperands(C.Structure):
                                           "rope_cos", "rope_sin", "pos", "rope_pairs", "key_pad")]
 
 
+class GemmParams(C.Structure):
+    """ZdrawGemmParams (metal_c.zig:276-283)"""
+    _fields_ = [("m", C.c_uint32), ("k", C.c_uint32), ("n", C.c_uint32), ("dtype", C.c_uint32),
+                ("mode", C.c_uint32), ("weight_offset", C.c_uint64)]
+
+
+class GemmExt(C.Structure):
+    """ZdrawHipGemmExt"""
+    _fields_ = [("a_off", C.c_uint64), ("c_off", C.c_uint64), ("lda", C.c_uint64), ("ldw", C.c_uint64),
+                ("ldc", C.c_uint64), ("a_dtype", C.c_uint32), ("c_dtype", C.c_uint32)]
+
+
+W_F16, W_BF16, W_F32 = 1, 2, 3     # weight dtype codes of GemmParams.dtype
+GEMM_EXACT, GEMM_HALF = 1, 2       # GemmParams.mode
+
 # every symbol include/zdraw_hip.h declares: name -> (restype, argtypes)
 _vp, _sz, _u32, _u64, _int = C.c_void_p, C.c_size_t, C.c_uint32, C.c_uint64, C.c_int
 _AP, _AX, _QO = C.POINTER(AttnParams), C.POINTER(AttnExt), C.POINTER(QkOperands)
+_GP, _GX = C.POINTER(GemmParams), C.POINTER(GemmExt)
 SYMBOLS = {
     "zdraw_hip_create_device": (_vp, []),
     "zdraw_hip_release_device": (None, [_vp]),
@@ -76,6 +92,11 @@ SYMBOLS = {
     "zdraw_hip_gpu_ns": (_u64, []),
     "zdraw_hip_trace_attention": (None, [_int]),
     "zdraw_hip_trace_attention_ns": (_u64, [C.POINTER(C.c_uint64)]),
+    "zdraw_hip_run_gemm": (_int, [_vp, _vp, _vp, _vp, _vp, _GP]),
+    "zdraw_hip_run_gemm_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _GP]),
+    "zdraw_hip_run_gemm_off_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _GP, _u64, _u64]),
+    "zdraw_hip_run_gemm_f16a_enc": (_int, [_vp, _vp, _vp, _vp, _GP, _u64, _u64]),
+    "zdraw_hip_run_gemm_ext_enc": (_int, [_vp, _vp, _vp, _vp, _GP, _GX]),
     "zdraw_hip_mfma_probe": (_int, [_int, _int, C.POINTER(C.c_double)]),
     "zdraw_hip_clock_probe": (None, [_int]),
     "zdraw_hip_clock_probe_read": (C.c_size_t, [C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_size_t]),
