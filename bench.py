@@ -99,8 +99,91 @@ def spin_up(L, ctx, res, ms):
     return n
 
 
+def gemm_main(args):
+    """`--path gemm`: the projection GEMM C[m][n] = A[m][k] x W[n][k]^T on its own (bf16 operands
+    and output, fp32 accumulation), by default the fused Q/K/V projection of a Klein 1024^2 block
+    (4608 tokens, hidden 3072 -> 3 x 3072). Same timing discipline as the attention line."""
+    import numpy as np
+
+    from zdraw_amd import hip, host
+
+    L = hip.lib()
+    ctx = host.Context.init()
+    m, k, n = args.m, args.k, args.n
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
+    ab, wb = ctx.buffer(host.f32_to_bf16_bits(a)), ctx.buffer(host.f32_to_bf16_bits(w))
+    cb = ctx.buffer(nbytes=m * n * 2)
+    params = hip.GemmParams(m, k, n, hip.W_BF16, hip.GEMM_HALF, 0)
+    ext = hip.GemmExt(0, 0, 0, 0, 0, hip.BF16, hip.BF16)
+
+    def burst(count):
+        b = L.zdraw_hip_batch_begin(ctx.queue)
+        for _ in range(count):
+            rc = L.zdraw_hip_run_gemm_ext_enc(b, ab.handle, wb.handle, cb.handle, C.byref(params), C.byref(ext))
+            if rc != 0:
+                raise RuntimeError(f"gemm rc={rc}: {hip.last_error()}")
+        if L.zdraw_hip_batch_end(b) != 0:
+            raise RuntimeError("batch_end failed")
+
+    t0 = time.perf_counter()
+    spun = 0
+    while (time.perf_counter() - t0) * 1e3 < args.spinup_ms:
+        burst(100)
+        spun += 100
+    burst(max(args.warmup, 1))
+    # HIP events on the library's stream around the K timed launches (no other kernel runs between them)
+    e0, e1 = L.zdraw_hip_event_create(), L.zdraw_hip_event_create()
+    L.zdraw_hip_queue_sync(ctx.queue)
+    t0 = time.perf_counter()
+    L.zdraw_hip_event_record(e0, ctx.queue)
+    burst(args.steps)
+    L.zdraw_hip_event_record(e1, ctx.queue)
+    L.zdraw_hip_event_sync(e1)
+    wall = time.perf_counter() - t0
+    kern_ms = L.zdraw_hip_event_elapsed_ms(e0, e1) / args.steps
+    out = host.bf16_bits_to_f32(cb.read(np.uint16, (m, n)))
+    if not np.isfinite(out).all():
+        raise RuntimeError("non-finite output")
+    flops = 2.0 * m * k * n
+    value = flops / (wall / args.steps) / 1e12
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+    line = {
+        "metric": "projection GEMM TFLOP/s + % of bf16 MFMA peak",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"gemm: C[{m}][{n}] = A[{m}][{k}] x W[{n}][{k}]^T, bf16 in and out, fp32 accumulate",
+                   "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS, "untimed_spinup_launches": spun},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "gemm_kernel", "kernel_ms": kern_ms},
+    }
+    if not args.no_cpu:
+        from oracle import zoracle as zo
+        rows = 16
+        t0 = time.perf_counter()
+        zo.linear_batch(a[:rows], w)
+        dt = time.perf_counter() - t0
+        rows = int(max(16, min(m, rows * 10.0 / max(dt, 1e-6))))
+        t0 = time.perf_counter()
+        zo.linear_batch(a[:rows], w)
+        dt = time.perf_counter() - t0
+        line["cpu_baseline"] = {"value": 2.0 * rows * k * n / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                                "sample": f"{rows} of {m} rows in {dt:.1f} s; full call extrapolates to {dt / rows * m:.0f} s"}
+    for b in (ab, wb, cb):
+        b.release()
+    ctx.deinit()
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--path", choices=["attention", "gemm"], default="attention",
+                    help="attention (the headline metric) or the projection GEMM beside it")
+    ap.add_argument("--m", type=int, default=4608)
+    ap.add_argument("--k", type=int, default=3072)
+    ap.add_argument("--n", type=int, default=9216)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
@@ -119,6 +202,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)")
+    if args.path == "gemm":
+        return gemm_main(args)
 
     import numpy as np
 

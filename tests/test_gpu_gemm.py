@@ -199,3 +199,67 @@ def test_reference_offset_entries_and_bit_stability(ctx, pipe):
     assert np.abs(outs[0][0] - want[0]).max() <= 2e-5 * s   # f16a_enc: first half, A already half
     for b in (ab, a16b, wb, cb):
         b.release()
+
+
+def test_single_block_chain_projection_attention_projection(ctx):
+    # The attention segment of a Klein single block (klein/zflux2_resident.zig:1986-2058):
+    # q, k, v = x W^T with W three row ranges of ONE fused weight (weight_offset selects them),
+    # written as bf16 token-major rows; QK-norm + rope + attention writes O into the first
+    # `hidden` columns of the concat operand (pitch hidden + inner); the out projection reads
+    # that operand whole. Checked against the oracle chain with the same bf16 hand-over points.
+    from tests import refimpl
+    from zdraw_amd import workloads as wl
+
+    L = hip.lib()
+    w = wl.by_name("klein_1024", seed=21, small=True)
+    tokens, heads = w.tokens, w.heads
+    hidden, inner = heads * 128, 2 * heads * 128
+    pitch = hidden + inner
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((tokens, hidden), dtype=np.float32)
+    w_qkv = rng.standard_normal((3 * hidden, hidden), dtype=np.float32) * np.float32(hidden ** -0.5)
+    w_out = rng.standard_normal((hidden, pitch), dtype=np.float32) * np.float32(pitch ** -0.5)
+    mlp = rng.standard_normal((tokens, inner), dtype=np.float32)
+    nq, nk = (1.0 + 0.1 * rng.standard_normal(128).astype(np.float32) for _ in range(2))
+    rb = lambda a: host.bf16_bits_to_f32(host.f32_to_bf16_bits(a))
+
+    xb, wqkvb, woutb = ctx.buffer(host.f32_to_bf16_bits(x)), ctx.buffer(host.f32_to_bf16_bits(w_qkv)), ctx.buffer(host.f32_to_bf16_bits(w_out))
+    qkv = [ctx.buffer(nbytes=tokens * hidden * 2) for _ in range(3)]
+    cat0 = np.zeros((tokens, pitch), np.uint16)
+    cat0[:, hidden:] = host.f32_to_bf16_bits(mlp)
+    cat = ctx.buffer(cat0)
+    out = ctx.buffer(nbytes=tokens * hidden * 4)
+    nqb, nkb = ctx.buffer(nq), ctx.buffer(nk)
+    cos, sin = ctx.buffer(w.rope_cos), ctx.buffer(w.rope_sin)
+
+    batch = L.zdraw_hip_batch_begin(ctx.queue)
+    ext = hip.GemmExt(0, 0, 0, 0, 0, hip.BF16, hip.BF16)
+    for i in range(3):
+        params = hip.GemmParams(tokens, hidden, hidden, hip.W_BF16, hip.GEMM_HALF, i * hidden * hidden * 2)
+        assert L.zdraw_hip_run_gemm_ext_enc(batch, xb.handle, wqkvb.handle, qkv[i].handle, C.byref(params), C.byref(ext)) == 0, hip.last_error()
+    assert L.zdraw_hip_batch_end(batch) == 0
+    ctx.joint_klein(qkv[0], qkv[1], qkv[2], cat, tokens=tokens, heads=heads, norm_q=nqb, norm_k=nkb,
+                    rope_cos=cos, rope_sin=sin, out_row_stride=pitch, k_site=hip.K_PREPASS,
+                    score_bound=host.score_bound(nq, nk, None, None))
+    batch = L.zdraw_hip_batch_begin(ctx.queue)
+    params = hip.GemmParams(tokens, pitch, hidden, hip.W_BF16, hip.GEMM_HALF, 0)
+    assert L.zdraw_hip_run_gemm_f16a_enc(batch, cat.handle, woutb.handle, out.handle, C.byref(params), 0, 0) == 0, hip.last_error()
+    assert L.zdraw_hip_batch_end(batch) == 0
+    got = out.read(np.float32, (tokens, hidden))
+
+    # oracle chain
+    xr, wr = rb(x), rb(w_qkv)
+    q, k, v = (rb(zo.linear_batch(xr, wr[i * hidden:(i + 1) * hidden])).reshape(tokens, heads, 128) for i in range(3))
+    c2, s2 = zo.klein_build_rope_ref(w.grid[0], w.grid[1], theta=w.theta, txt_len=w.txt_len)
+    qn = zo.klein_apply_rope(zo.klein_rms_norm_heads(q, nq), c2, s2)
+    kn = zo.klein_apply_rope(zo.klein_rms_norm_heads(k, nk), c2, s2)
+    o = zo.attention_run(qn, kn, v, zo.Config(tokens, heads, heads, 128)).reshape(tokens, hidden)
+    catr = np.concatenate([rb(o), rb(mlp)], axis=1)
+    want = zo.linear_batch(catr, rb(w_out))
+    # q, k, v and O each pass through a bf16 hand-over whose rounding can flip on a last-bit
+    # difference, so the bar is the attention path's: 2e-2 max / 2e-3 mean in units of the output scale
+    s = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    err = np.abs(got - want)
+    assert err.max() <= 2e-2 * max(s, 1.0) and err.mean() <= 2e-3 * max(s, 1.0), (err.max(), err.mean(), s)
+    for b in [xb, wqkvb, woutb, cat, out, nqb, nkb, cos, sin] + qkv:
+        b.release()

@@ -134,11 +134,21 @@ __global__ void __launch_bounds__(NT, 2) gemm_kernel(const GemmArgs g) {
     };
     auto store_slab = [&](int s) __attribute__((always_inline)) {
         unsigned short* st = lds + (s & 1) * STAGE_ELEMS;
-        const bool keep = s * BK + kc * 8 < g.k; // chunks past k (last slab only) contribute zeros
+        // chunks past k contribute zeros; only the last slab of a k that is not a multiple of 64 has any
+        const bool ragged = (s + 1) * BK > g.k; // wave-uniform
+        const bool keep = !ragged || s * BK + kc * 8 < g.k;
+        if (ragged) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            *reinterpret_cast<u32x4*>(st + (lr + 64 * j) * PITCH + kc * 8) = to_half8<TA, F16>(ra[j], keep);
-            *reinterpret_cast<u32x4*>(st + (BM + lr + 64 * j) * PITCH + kc * 8) = to_half8<unsigned short, F16>(rw[j], keep);
+            for (int j = 0; j < 4; j++) {
+                *reinterpret_cast<u32x4*>(st + (lr + 64 * j) * PITCH + kc * 8) = to_half8<TA, F16>(ra[j], keep);
+                *reinterpret_cast<u32x4*>(st + (BM + lr + 64 * j) * PITCH + kc * 8) = to_half8<unsigned short, F16>(rw[j], keep);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                *reinterpret_cast<u32x4*>(st + (lr + 64 * j) * PITCH + kc * 8) = to_half8<TA, F16>(ra[j], true);
+                *reinterpret_cast<u32x4*>(st + (BM + lr + 64 * j) * PITCH + kc * 8) = to_half8<unsigned short, F16>(rw[j], true);
+            }
         }
     };
 
@@ -172,9 +182,13 @@ __global__ void __launch_bounds__(NT, 2) gemm_kernel(const GemmArgs g) {
                 for (int j = 0; j < 4; j++) acc[i][j] = mfma<F16>(af[i], wf[j], acc[i][j]);
             if (kk == 0) {
                 // slab s+1 (in registers since the previous iteration) goes to the other stage,
-                // whose readers finished before the last barrier; then slab s+2 starts loading
+                // whose readers finished before the last barrier; then slab s+2 starts loading.
+                // The fences keep the loads here: sunk to the end of the iteration they would
+                // be waited for as soon as they are issued.
+                __builtin_amdgcn_sched_barrier(0);
                 store_slab(s + 1);
                 load_slab(s + 2);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         __syncthreads();
