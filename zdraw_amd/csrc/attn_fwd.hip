@@ -41,6 +41,9 @@ namespace fwd {
 #ifndef ZDRAW_MFMA_PRIO
 #define ZDRAW_MFMA_PRIO 1     // wave priority while an MFMA is issued (0 = leave it alone)
 #endif
+#ifndef ZDRAW_DIRECT_LDS
+#define ZDRAW_DIRECT_LDS 1    // prepared bf16 K/V blocks go from global memory straight into LDS
+#endif
 #ifndef ZDRAW_STORE_SLOT
 #define ZDRAW_STORE_SLOT 1    // slot after which a step moves its staged block into the ring
 #endif
@@ -105,15 +108,25 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     constexpr int TPK = 16 / CPT;     // threads sharing one key row
     constexpr int NST = ring_stages(QB, NW);
     constexpr bool XSTEP = NST == 8;          // fragment reads run ahead across step boundaries
-    constexpr int AHEAD = NST == 8 ? 4 : 2;   // a block is stored AHEAD steps before S needs its K
+    // Prepared bf16 operands with every block full (K pre-pass mode, no mask) skip the
+    // registers: each wave moves four K rows and four V rows of a block from global
+    // memory straight into the ring (buffer_load ... lds). Such a load puts lane i's
+    // 16 bytes at base + 16 i, so rows are 256 bytes without padding and bank
+    // conflicts are avoided by swizzling the 16-byte chunk position instead:
+    // K chunk c of row r sits at c ^ (r & 15), V chunk c of row r at c ^ ((r & 3) << 2).
+    constexpr bool DMA = ZDRAW_DIRECT_LDS && std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && !MASKED && NW == 8 && QB == 1;
+    constexpr int KSTAGE = DMA ? KB * D : KS_ELEMS; // elements per ring stage
+    constexpr int VSTAGE = DMA ? KB * D : VS_ELEMS;
+    // a block enters the ring AHEAD steps before S needs its K (direct loads: one more step, to land)
+    constexpr int AHEAD = NST == 8 ? (DMA ? 5 : 4) : 2;
     constexpr int LA = ZDRAW_LDS_LOOKAHEAD;   // slots between an LDS fragment read and its MFMA
     constexpr int RB = ZDRAW_READ_BATCH;      // slots whose reads are issued together (divides 16 and LA)
     constexpr int MFMA_PRIO = ZDRAW_MFMA_PRIO; // wave priority while an MFMA is being issued
     constexpr int STORE_SLOT = ZDRAW_STORE_SLOT; // slot after which the ring store is issued
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* const Ks = reinterpret_cast<bf16_t*>(smem);
-    bf16_t* const Vs = Ks + NST * KS_ELEMS;
-    unsigned short* const blocks = reinterpret_cast<unsigned short*>(Vs + NST * VS_ELEMS);
+    bf16_t* const Vs = Ks + NST * KSTAGE;
+    unsigned short* const blocks = reinterpret_cast<unsigned short*>(Vs + NST * VSTAGE);
     __shared__ int s_nblocks;
 
     unsigned long long clk_c0 = 0, clk_r0 = 0;
@@ -147,8 +160,8 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // that stage must hold finite numbers, so it is zeroed. (The last S update
     // reads a K stage past the end; its result is discarded.)
     {
-        u32x4* z = reinterpret_cast<u32x4*>(Vs + (NST - 1) * VS_ELEMS);
-        constexpr int n16 = (int)(VS_ELEMS * sizeof(bf16_t) / 16);
+        u32x4* z = reinterpret_cast<u32x4*>(Vs + (NST - 1) * VSTAGE);
+        constexpr int n16 = (int)(VSTAGE * sizeof(bf16_t) / 16);
         for (int i = tid; i < n16; i += NT) z[i] = u32x4{0u, 0u, 0u, 0u};
     }
 
@@ -304,6 +317,21 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         for (int c = 0; c < CPT; c++) *reinterpret_cast<u32x4*>(vdst + 8 * c) = raw_to_bf16(r.vraw[c]);
     };
 
+    // Direct path: wave w moves rows 4 w + lane / 16 of block position i into ring stage
+    // i % NST; the lane that fills chunk position p of row r fetches the chunk that the
+    // swizzle places there. (Every block is full in this build: no tail offsets.)
+    const int dma_row = 4 * wave + (lane >> 4);
+    const unsigned dma_k_off = ((unsigned)dma_row * (unsigned)a.k_ts + (unsigned)(((lane & 15) ^ (dma_row & 15)) * 8)) * 2u;
+    const unsigned dma_v_off = ((unsigned)dma_row * (unsigned)a.v_ts + (unsigned)(((lane & 15) ^ ((dma_row & 3) << 2)) * 8)) * 2u;
+    const u32x4 dma_k_rsrc = make_rsrc_words(reinterpret_cast<const TIn*>(a.k) + (int64_t)seg * a.k_bs + (int64_t)head * a.k_hs, k_span);
+    const u32x4 dma_v_rsrc = make_rsrc_words(reinterpret_cast<const TIn*>(a.v) + (int64_t)seg * a.v_bs + (int64_t)head * a.v_hs, v_span);
+    auto dma_fetch = [&](int i) __attribute__((always_inline)) {
+        const int ii = i < nblk ? i : nblk - 1; // past the end: a harmless re-fetch into a dead stage
+        const int stage = i & (NST - 1);
+        load_to_lds_16(dma_k_rsrc, Ks + stage * KSTAGE + 4 * wave * D, dma_k_off, (unsigned)ii * k_blk_bytes);
+        load_to_lds_16(dma_v_rsrc, Vs + stage * VSTAGE + 4 * wave * D, dma_v_off, (unsigned)ii * v_blk_bytes);
+    };
+
     // ---- running state
     f32x16 oacc[QB][4]; // O^T: lane query 32*qi + l32, dims 32*blk + 8i + 4h + j
 #pragma unroll
@@ -319,16 +347,29 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         l_run[qi] = 0.f;
     }
 
+    // LDS addresses of this lane's fragments. K: key row l32, dims 16 s + 8 h .. +7.
+    // V: the 4 x 16 patch of the transposing read (row 16 kb + 8 half + 4 h + tr_row).
+    const int tr_row = (lane & 15) >> 2;
+    const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    auto k_frag = [&](int stage, int s) __attribute__((always_inline)) -> const bf16_t* {
+        if constexpr (DMA) return Ks + stage * KSTAGE + l32 * D + (((2 * s + h) ^ (l32 & 15)) * 8);
+        else return Ks + stage * KSTAGE + l32 * KPITCH + 8 * h + 16 * s;
+    };
+    auto v_frag = [&](int stage, int kb, int blk, int half) __attribute__((always_inline)) -> const bf16_t* {
+        const int row = 16 * kb + 8 * half + 4 * h + tr_row;
+        if constexpr (DMA) return Vs + stage * VSTAGE + row * D + ((blk ^ tr_row) * 32) + tr_col; // row & 3 == tr_row
+        else return Vs + stage * VSTAGE + row * VPITCH + 32 * blk + tr_col;
+    };
+
     // S^T block = K(block) . Q^T for both query blocks
     auto qk_block = [&](int stage, f32x16 (&s_out)[QB]) {
 #pragma unroll
         for (int qi = 0; qi < QB; qi++)
 #pragma unroll
             for (int j = 0; j < 16; j++) s_out[qi][j] = 0.f;
-        const bf16_t* kt = Ks + stage * KS_ELEMS + l32 * KPITCH + 8 * h;
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kt + 16 * s);
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(k_frag(stage, s));
 #pragma unroll
             for (int qi = 0; qi < QB; qi++)
                 s_out[qi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qi][s], s_out[qi], 0, 0, 0);
@@ -336,16 +377,13 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     };
 
     // O^T += V(block)^T . P^T
-    const int tr_row = (lane & 15) >> 2;
-    const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     auto pv_block = [&](int stage, const bf16x8 (&p)[QB][2]) {
-        const bf16_t* vt = Vs + stage * VS_ELEMS + (4 * h + tr_row) * VPITCH + tr_col;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
             for (int blk = 0; blk < 4; blk++) {
-                const s16x4 lo = lds_read_tr(vt + (16 * kb) * VPITCH + 32 * blk);
-                const s16x4 hi = lds_read_tr(vt + (16 * kb + 8) * VPITCH + 32 * blk);
+                const s16x4 lo = lds_read_tr(v_frag(stage, kb, blk, 0));
+                const s16x4 hi = lds_read_tr(v_frag(stage, kb, blk, 1));
                 typedef short s16x8 __attribute__((ext_vector_type(8)));
                 const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
@@ -365,13 +403,12 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // 16*(slot/2).., odd slots read the V(bb-1) patch for output block (slot/2)%4, keys 16*(slot/8)..
     auto frag_read = [&](int bb, int slot) __attribute__((always_inline)) {
         if (slot & 1) {
-            const bf16_t* vt = Vs + ((bb + NST - 1) & (NST - 1)) * VS_ELEMS + (4 * h + tr_row) * VPITCH + tr_col;
             const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
-            vlo[idx] = lds_read_tr(vt + (16 * kb) * VPITCH + 32 * blk);
-            vhi[idx] = lds_read_tr(vt + (16 * kb + 8) * VPITCH + 32 * blk);
+            const int stage = (bb + NST - 1) & (NST - 1);
+            vlo[idx] = lds_read_tr(v_frag(stage, kb, blk, 0));
+            vhi[idx] = lds_read_tr(v_frag(stage, kb, blk, 1));
         } else {
-            const bf16_t* kt = Ks + ((bb + 1) & (NST - 1)) * KS_ELEMS + l32 * KPITCH + 8 * h;
-            kf[slot >> 1] = *reinterpret_cast<const bf16x8*>(kt + 16 * (slot >> 1));
+            kf[slot >> 1] = *reinterpret_cast<const bf16x8*>(k_frag((bb + 1) & (NST - 1), slot >> 1));
         }
     };
 
@@ -522,8 +559,12 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             // ring: block b+AHEAD (in this register set since two steps ago) goes to its stage,
             // whose previous tenant's last reader (V, NST-AHEAD-1 steps back) is at least one
             // barrier behind; then the set starts loading block b+AHEAD+2
-            if (g == STORE_SLOT) stage_store(regs, (b + AHEAD) & (NST - 1));
-            if (g == STORE_SLOT + 1) stage_load(regs, b + AHEAD + 2);
+            if constexpr (DMA) {
+                if (g == STORE_SLOT) dma_fetch(b + AHEAD);
+            } else {
+                if (g == STORE_SLOT) stage_store(regs, (b + AHEAD) & (NST - 1));
+                if (g == STORE_SLOT + 1) stage_load(regs, b + AHEAD + 2);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
 
@@ -543,6 +584,9 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 // wave complete in order and every read of this step has been consumed, so
                 // this step's ring writes are complete: the bare barrier orders them.
                 asm volatile("" ::: "memory");
+                // direct loads: all but this step's two must have landed (vmcnt(2)); a block is
+                // first read two barriers after it was requested
+                if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0x0F72);
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
             } else {
@@ -553,7 +597,11 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 
     if (nblk > 0) {
         // prologue: blocks 0 .. AHEAD-1 into the ring, blocks AHEAD and AHEAD+1 in flight
-        {
+        if constexpr (DMA) {
+#pragma unroll
+            for (int i = 0; i < AHEAD; i++) dma_fetch(i);
+            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+        } else {
             StageRegs pre[AHEAD];
 #pragma unroll
             for (int i = 0; i < AHEAD; i++) stage_load(pre[i], i);
@@ -592,6 +640,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         } else {
             pv_block((nblk - 1) & (NST - 1), p_a);
         }
+        if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
     }
 
     // ---- epilogue: O = O^T / l
