@@ -63,7 +63,8 @@ constexpr float kTau = 8.0f;             // log2 headroom of the lazy softmax ma
 // ahead, one barrier per step).
 constexpr int ring_stages(int qb, int nw) { return (qb == 2 || nw == 8) ? 8 : 4; }
 constexpr size_t lds_bytes(int nst) {
-    return (size_t)nst * (KS_ELEMS + VS_ELEMS) * sizeof(bf16_t) + (size_t)MAX_BLOCKS * sizeof(unsigned short);
+    // ring + key-block list (u16) + per-block exclusion masks (u32)
+    return (size_t)nst * (KS_ELEMS + VS_ELEMS) * sizeof(bf16_t) + (size_t)MAX_BLOCKS * (sizeof(unsigned short) + sizeof(unsigned));
 }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -108,13 +109,12 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     constexpr int TPK = 16 / CPT;     // threads sharing one key row
     constexpr int NST = ring_stages(QB, NW);
     constexpr bool XSTEP = NST == 8;          // fragment reads run ahead across step boundaries
-    // Prepared bf16 operands with every block full (K pre-pass mode, no mask) skip the
-    // registers: each wave moves four K rows and four V rows of a block from global
+    // Prepared bf16 operands (K pre-pass mode) skip the registers: each wave moves four K rows and four V rows of a block from global
     // memory straight into the ring (buffer_load ... lds). Such a load puts lane i's
     // 16 bytes at base + 16 i, so rows are 256 bytes without padding and bank
     // conflicts are avoided by swizzling the 16-byte chunk position instead:
     // K chunk c of row r sits at c ^ (r & 15), V chunk c of row r at c ^ ((r & 3) << 2).
-    constexpr bool DMA = ZDRAW_DIRECT_LDS && std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && !MASKED && NW == 8 && QB == 1;
+    constexpr bool DMA = ZDRAW_DIRECT_LDS && std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && NW == 8 && QB == 1;
     constexpr int KSTAGE = DMA ? KB * D : KS_ELEMS; // elements per ring stage
     constexpr int VSTAGE = DMA ? KB * D : VS_ELEMS;
     // a block enters the ring AHEAD steps before S needs its K (direct loads: one more step, to land)
@@ -127,6 +127,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     bf16_t* const Ks = reinterpret_cast<bf16_t*>(smem);
     bf16_t* const Vs = Ks + NST * KSTAGE;
     unsigned short* const blocks = reinterpret_cast<unsigned short*>(Vs + NST * VSTAGE);
+    unsigned* const bmask = reinterpret_cast<unsigned*>(blocks + MAX_BLOCKS); // bit j: key j of the block is excluded
     __shared__ int s_nblocks;
 
     unsigned long long clk_c0 = 0, clk_r0 = 0;
@@ -169,25 +170,33 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     const int nb_all = (a.key_limit + KB - 1) / KB;
     const unsigned char* const kp = a.key_pad ? a.key_pad + (int64_t)seg * a.mask_bs : nullptr;
     int nblk = nb_all;
-    if (MASKED && kp) {
-        if (wave == 0) {
-            int count = 0;
-            for (int base = 0; base < nb_all; base += 64) {
-                const int t = base + lane;
-                bool act = false;
-                if (t < nb_all) {
-                    const int k0 = t * KB;
-                    const int k1 = min(k0 + KB, a.key_limit);
-                    for (int j = k0; j < k1; j++) act |= (kp[j] == 0);
-                }
-                const unsigned long long m = __ballot(act);
-                if (act) blocks[count + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short)t;
-                count += __popcll(m);
+    if constexpr (MASKED) {
+        // exclusion mask of every key block (padding mask, key limit, tail), two blocks per wave pass
+        for (int t2 = wave; 2 * t2 < nb_all; t2 += NW) {
+            const int key = t2 * 64 + lane;
+            const bool bad = key >= a.key_limit || (kp != nullptr && kp[key < a.key_limit ? key : 0] != 0);
+            const unsigned long long m = __ballot(bad);
+            if (lane == 0) {
+                bmask[2 * t2] = (unsigned)m;
+                if (2 * t2 + 1 < MAX_BLOCKS) bmask[2 * t2 + 1] = (unsigned)(m >> 32);
             }
-            if (lane == 0) s_nblocks = count;
         }
         __syncthreads();
-        nblk = __builtin_amdgcn_readfirstlane(s_nblocks);
+        if (kp) { // compact the blocks that admit at least one key
+            if (wave == 0) {
+                int count = 0;
+                for (int base = 0; base < nb_all; base += 64) {
+                    const int t = base + lane;
+                    const bool act = t < nb_all && bmask[t < nb_all ? t : 0] != 0xffffffffu;
+                    const unsigned long long m = __ballot(act);
+                    if (act) blocks[count + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short)t;
+                    count += __popcll(m);
+                }
+                if (lane == 0) s_nblocks = count;
+            }
+            __syncthreads();
+            nblk = __builtin_amdgcn_readfirstlane(s_nblocks);
+        }
     }
     // wave-uniform by construction; readfirstlane lets the compiler keep it in scalar registers
     auto block_of = [&](int i) -> int { return (MASKED && kp) ? __builtin_amdgcn_readfirstlane((int)blocks[i]) : i; };
@@ -319,17 +328,30 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 
     // Direct path: wave w moves rows 4 w + lane / 16 of block position i into ring stage
     // i % NST; the lane that fills chunk position p of row r fetches the chunk that the
-    // swizzle places there. (Every block is full in this build: no tail offsets.)
+    // swizzle places there. In the block that holds the last row, rows past the sequence
+    // re-read the last row (they are masked before the softmax).
     const int dma_row = 4 * wave + (lane >> 4);
-    const unsigned dma_k_off = ((unsigned)dma_row * (unsigned)a.k_ts + (unsigned)(((lane & 15) ^ (dma_row & 15)) * 8)) * 2u;
-    const unsigned dma_v_off = ((unsigned)dma_row * (unsigned)a.v_ts + (unsigned)(((lane & 15) ^ ((dma_row & 3) << 2)) * 8)) * 2u;
+    const unsigned dma_k_chunk = (unsigned)(((lane & 15) ^ (dma_row & 15)) * 8);
+    const unsigned dma_v_chunk = (unsigned)(((lane & 15) ^ ((dma_row & 3) << 2)) * 8);
+    const unsigned dma_k_off = ((unsigned)dma_row * (unsigned)a.k_ts + dma_k_chunk) * 2u;
+    const unsigned dma_v_off = ((unsigned)dma_row * (unsigned)a.v_ts + dma_v_chunk) * 2u;
+    const int dma_tail_row = min(dma_row, last_row - last_blk * KB);
+    const unsigned dma_k_off_tail = ((unsigned)dma_tail_row * (unsigned)a.k_ts + dma_k_chunk) * 2u;
+    const unsigned dma_v_off_tail = ((unsigned)dma_tail_row * (unsigned)a.v_ts + dma_v_chunk) * 2u;
     const u32x4 dma_k_rsrc = make_rsrc_words(reinterpret_cast<const TIn*>(a.k) + (int64_t)seg * a.k_bs + (int64_t)head * a.k_hs, k_span);
     const u32x4 dma_v_rsrc = make_rsrc_words(reinterpret_cast<const TIn*>(a.v) + (int64_t)seg * a.v_bs + (int64_t)head * a.v_hs, v_span);
     auto dma_fetch = [&](int i) __attribute__((always_inline)) {
         const int ii = i < nblk ? i : nblk - 1; // past the end: a harmless re-fetch into a dead stage
         const int stage = i & (NST - 1);
-        load_to_lds_16(dma_k_rsrc, Ks + stage * KSTAGE + 4 * wave * D, dma_k_off, (unsigned)ii * k_blk_bytes);
-        load_to_lds_16(dma_v_rsrc, Vs + stage * VSTAGE + 4 * wave * D, dma_v_off, (unsigned)ii * v_blk_bytes);
+        const int blk = block_of(ii);
+        unsigned ko = dma_k_off, vo = dma_v_off;
+        if constexpr (MASKED) {
+            const bool tail = blk >= last_blk; // wave-uniform
+            ko = tail ? dma_k_off_tail : dma_k_off;
+            vo = tail ? dma_v_off_tail : dma_v_off;
+        }
+        load_to_lds_16(dma_k_rsrc, Ks + stage * KSTAGE + 4 * wave * D, ko, (unsigned)blk * k_blk_bytes);
+        load_to_lds_16(dma_v_rsrc, Vs + stage * VSTAGE + 4 * wave * D, vo, (unsigned)blk * v_blk_bytes);
     };
 
     // ---- running state
@@ -412,6 +434,11 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         }
     };
 
+    unsigned badm_cur = 0; // exclusion mask of the block whose scores the next step exponentiates
+    if constexpr (MASKED) {
+        if (nblk > 0) badm_cur = bmask[block_of(0)];
+    }
+
     // One pipeline step for list position b: consumes S(b) and P(b-1),
     // produces S(b+1) and P(b). The three streams are independent, so the
     // step is laid out by hand as 16 slots, each fenced from the next:
@@ -442,18 +469,18 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 
         if constexpr (MASKED) {
             // excluded keys (padding mask, key limit, tail) -> -inf; bit kk of badm = key kk of the block
-            const int key = block_of(b) * KB + l32;
-            const bool bad = key >= a.key_limit || (kp != nullptr && kp[key < a.key_limit ? key : 0] != 0);
-            const unsigned badm = (unsigned)__ballot(bad); // lanes 0..31 carry the block's 32 keys
+            const unsigned badm = __builtin_amdgcn_readfirstlane(badm_cur); // fetched from LDS during the previous step
+            if (badm != 0u) { // wave-uniform: most blocks exclude nothing
 #pragma unroll
-            for (int qi = 0; qi < QB; qi++)
+                for (int qi = 0; qi < QB; qi++)
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                    for (int i = 0; i < 4; i++)
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const int kk = 8 * i + 4 * h + j;
-                        s_cur[qi][4 * i + j] = ((badm >> kk) & 1u) ? -INFINITY : s_cur[qi][4 * i + j];
-                    }
+                        for (int j = 0; j < 4; j++) {
+                            const int kk = 8 * i + 4 * h + j;
+                            s_cur[qi][4 * i + j] = ((badm >> kk) & 1u) ? -INFINITY : s_cur[qi][4 * i + j];
+                        }
+            }
         }
 #pragma unroll
         for (int qi = 0; qi < QB; qi++)
@@ -559,6 +586,9 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             // ring: block b+AHEAD (in this register set since two steps ago) goes to its stage,
             // whose previous tenant's last reader (V, NST-AHEAD-1 steps back) is at least one
             // barrier behind; then the set starts loading block b+AHEAD+2
+            if constexpr (MASKED) {
+                if (g == 10) badm_cur = bmask[block_of(b + 1 < nblk ? b + 1 : nblk - 1)];
+            }
             if constexpr (DMA) {
                 if (g == STORE_SLOT) dma_fetch(b + AHEAD);
             } else {
