@@ -64,7 +64,7 @@ __device__ __forceinline__ Raw8<T> ld_raw8_buf(rsrc_t rsrc, unsigned thread_off,
 }
 
 // 16 bytes per lane from global memory straight into LDS: lane i's data lands at
-// lds_base + 16 i (lds_base, the descriptor and uniform_off are wave-uniform). The
+// lds_addr + 16 i (lds_addr, the descriptor and uniform_off are wave-uniform). The
 // instruction is written out so that the compiler does not make every later LDS
 // read wait for it; the CALLER orders it against those reads (s_waitcnt vmcnt +
 // barrier before the data is read, a barrier after the last read of what it overwrites).
@@ -72,9 +72,11 @@ __device__ __forceinline__ u32x4 make_rsrc_words(const void* base, unsigned byte
     const unsigned long long p = reinterpret_cast<unsigned long long>(base);
     return u32x4{(unsigned)p, (unsigned)(p >> 32) & 0xffffu, bytes, 0x00020000u};
 }
-__device__ __forceinline__ void load_to_lds_16(u32x4 rsrc, const void* lds_base, unsigned thread_off, unsigned uniform_off) {
-    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
-        (unsigned)(unsigned long long)(__attribute__((address_space(3))) const void*)lds_base);
+// LDS byte address of a __shared__ object (taken once; the cast carries a null check).
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    return (unsigned)(unsigned long long)(__attribute__((address_space(3))) const void*)p;
+}
+__device__ __forceinline__ void load_to_lds_16(u32x4 rsrc, unsigned lds_addr, unsigned thread_off, unsigned uniform_off) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(thread_off), "s"(rsrc), "s"(uniform_off)

@@ -80,14 +80,10 @@ __device__ __forceinline__ void pin(T& v) {
     asm volatile("" : "+v"(v));
 }
 
-// Four keys (rows) for this lane's head-dim column, from row-major V in LDS.
-// Within each 16-lane group the hardware returns to lane i, element j, the
-// value at (row of source lane (i>>2)+4j, column i&3 of that lane's 4-element
-// chunk); `p` must point at row (lane&15)>>2, chunk lane&3 of the 4x16 patch.
-__device__ __forceinline__ s16x4 lds_read_tr(const bf16_t* p) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(p)));
-}
+// The transposing LDS read ds_read_b64_tr_b16 (used for V below): within each 16-lane
+// group the hardware returns to lane i, element j, the value at (row of source lane
+// (i>>2)+4j, column i&3 of that lane's 4-element chunk); a lane's address must point at
+// row (lane&15)>>2, chunk lane&3 of the 4 x 16 patch.
 
 // QB = 32-query blocks per wave, NW = waves per workgroup. Built shapes:
 //   QB=1, NW=8: two waves per SIMD, 256 registers each (default);
@@ -340,9 +336,11 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     const unsigned dma_v_off_tail = ((unsigned)dma_tail_row * (unsigned)a.v_ts + dma_v_chunk) * 2u;
     const u32x4 dma_k_rsrc = make_rsrc_words(reinterpret_cast<const TIn*>(a.k) + (int64_t)seg * a.k_bs + (int64_t)head * a.k_hs, k_span);
     const u32x4 dma_v_rsrc = make_rsrc_words(reinterpret_cast<const TIn*>(a.v) + (int64_t)seg * a.v_bs + (int64_t)head * a.v_hs, v_span);
-    auto dma_fetch = [&](int i) __attribute__((always_inline)) {
+    // LDS byte addresses of this wave's four rows in stage 0 of the K ring and of the V ring
+    const unsigned dma_k_lds = __builtin_amdgcn_readfirstlane(lds_address(Ks) + (unsigned)(4 * wave * D * 2));
+    const unsigned dma_v_lds = __builtin_amdgcn_readfirstlane(lds_address(Vs) + (unsigned)(4 * wave * D * 2));
+    auto dma_fetch = [&](int i, int stage) __attribute__((always_inline)) {
         const int ii = i < nblk ? i : nblk - 1; // past the end: a harmless re-fetch into a dead stage
-        const int stage = i & (NST - 1);
         const int blk = block_of(ii);
         unsigned ko = dma_k_off, vo = dma_v_off;
         if constexpr (MASKED) {
@@ -350,8 +348,8 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             ko = tail ? dma_k_off_tail : dma_k_off;
             vo = tail ? dma_v_off_tail : dma_v_off;
         }
-        load_to_lds_16(dma_k_rsrc, Ks + stage * KSTAGE + 4 * wave * D, ko, (unsigned)blk * k_blk_bytes);
-        load_to_lds_16(dma_v_rsrc, Vs + stage * VSTAGE + 4 * wave * D, vo, (unsigned)blk * v_blk_bytes);
+        load_to_lds_16(dma_k_rsrc, dma_k_lds + (unsigned)stage * (KSTAGE * 2u), ko, (unsigned)blk * k_blk_bytes);
+        load_to_lds_16(dma_v_rsrc, dma_v_lds + (unsigned)stage * (VSTAGE * 2u), vo, (unsigned)blk * v_blk_bytes);
     };
 
     // ---- running state
@@ -369,18 +367,32 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         l_run[qi] = 0.f;
     }
 
-    // LDS addresses of this lane's fragments. K: key row l32, dims 16 s + 8 h .. +7.
-    // V: the 4 x 16 patch of the transposing read (row 16 kb + 8 half + 4 h + tr_row).
+    // LDS byte addresses of this lane's fragments in ring stage 0; a stage, a key half (kb)
+    // and a row half add constants. K: key row l32, dims 16 s + 8 h .. +7 (8 addresses, the
+    // swizzle makes them differ by more than a constant). V: the 4 x 16 patch of the
+    // transposing read, row 16 kb + 8 half + 4 h + tr_row, one address per output block.
     const int tr_row = (lane & 15) >> 2;
     const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    auto k_frag = [&](int stage, int s) __attribute__((always_inline)) -> const bf16_t* {
-        if constexpr (DMA) return Ks + stage * KSTAGE + l32 * D + (((2 * s + h) ^ (l32 & 15)) * 8);
-        else return Ks + stage * KSTAGE + l32 * KPITCH + 8 * h + 16 * s;
+    constexpr int KROW = DMA ? D : KPITCH, VROW = DMA ? D : VPITCH; // elements per LDS row
+    unsigned kfo[8], vfo[4];
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        const int col = DMA ? (((2 * s + h) ^ (l32 & 15)) * 8) : (8 * h + 16 * s);
+        kfo[s] = lds_address(Ks) + (unsigned)((l32 * KROW + col) * 2);
+    }
+#pragma unroll
+    for (int blk = 0; blk < 4; blk++) {
+        const int col = (DMA ? ((blk ^ tr_row) * 32) : (32 * blk)) + tr_col; // (4 h + tr_row) & 3 == tr_row
+        vfo[blk] = lds_address(Vs) + (unsigned)(((4 * h + tr_row) * VROW + col) * 2);
+    }
+    typedef const __attribute__((address_space(3))) bf16x8* lds_bf16x8_t;
+    typedef __attribute__((address_space(3))) s16x4* lds_s16x4_t;
+    auto k_frag = [&](int stage, int s) __attribute__((always_inline)) -> bf16x8 {
+        return *(lds_bf16x8_t)(kfo[s] + (unsigned)(stage * (KSTAGE * 2)));
     };
-    auto v_frag = [&](int stage, int kb, int blk, int half) __attribute__((always_inline)) -> const bf16_t* {
-        const int row = 16 * kb + 8 * half + 4 * h + tr_row;
-        if constexpr (DMA) return Vs + stage * VSTAGE + row * D + ((blk ^ tr_row) * 32) + tr_col; // row & 3 == tr_row
-        else return Vs + stage * VSTAGE + row * VPITCH + 32 * blk + tr_col;
+    auto v_frag = [&](int stage, int kb, int blk, int half) __attribute__((always_inline)) -> s16x4 {
+        return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_s16x4_t)(vfo[blk] + (unsigned)(stage * (VSTAGE * 2) + (16 * kb + 8 * half) * (VROW * 2))));
     };
 
     // S^T block = K(block) . Q^T for both query blocks
@@ -391,7 +403,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             for (int j = 0; j < 16; j++) s_out[qi][j] = 0.f;
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(k_frag(stage, s));
+            const bf16x8 kf = k_frag(stage, s);
 #pragma unroll
             for (int qi = 0; qi < QB; qi++)
                 s_out[qi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qi][s], s_out[qi], 0, 0, 0);
@@ -404,8 +416,8 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
             for (int blk = 0; blk < 4; blk++) {
-                const s16x4 lo = lds_read_tr(v_frag(stage, kb, blk, 0));
-                const s16x4 hi = lds_read_tr(v_frag(stage, kb, blk, 1));
+                const s16x4 lo = v_frag(stage, kb, blk, 0);
+                const s16x4 hi = v_frag(stage, kb, blk, 1);
                 typedef short s16x8 __attribute__((ext_vector_type(8)));
                 const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
@@ -423,14 +435,14 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     s16x4 vlo[8], vhi[8];
     // LDS fragment read for slot `slot` of step `bb`: even slots read K(bb+1) dims
     // 16*(slot/2).., odd slots read the V(bb-1) patch for output block (slot/2)%4, keys 16*(slot/8)..
-    auto frag_read = [&](int bb, int slot) __attribute__((always_inline)) {
+    // (k_stage holds K(bb+1), v_stage holds V(bb-1))
+    auto frag_read = [&](int k_stage, int v_stage, int slot) __attribute__((always_inline)) {
         if (slot & 1) {
             const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
-            const int stage = (bb + NST - 1) & (NST - 1);
-            vlo[idx] = lds_read_tr(v_frag(stage, kb, blk, 0));
-            vhi[idx] = lds_read_tr(v_frag(stage, kb, blk, 1));
+            vlo[idx] = v_frag(v_stage, kb, blk, 0);
+            vhi[idx] = v_frag(v_stage, kb, blk, 1);
         } else {
-            kf[slot >> 1] = *reinterpret_cast<const bf16x8*>(k_frag((bb + 1) & (NST - 1), slot >> 1));
+            kf[slot >> 1] = k_frag(k_stage, slot >> 1);
         }
     };
 
@@ -447,8 +459,24 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // Even slots extend S(b+1) = K(b+1) Q^T, odd slots add V(b-1)^T P(b-1)^T to O^T.
     // With the 8-stage ring the reads for the first LA slots of step b+1 are
     // issued in the last LA slots of step b, so no step starts by waiting on LDS.
-    auto step = [&](int b, StageRegs& regs, bool sync, f32x16 (&s_cur)[QB], f32x16 (&s_next)[QB], const bf16x8 (&p_prev)[QB][2],
-                    bf16x8 (&p_cur)[QB][2]) __attribute__((always_inline)) {
+    // `phase` is b modulo the ring depth as a compile-time constant (every LDS address of
+    // the step is then a register plus an immediate), or -1 when only b itself is known.
+    auto step = [&](auto phase, int b, StageRegs& regs, bool sync, f32x16 (&s_cur)[QB], f32x16 (&s_next)[QB],
+                    const bf16x8 (&p_prev)[QB][2], bf16x8 (&p_cur)[QB][2]) __attribute__((always_inline)) {
+        constexpr int J = decltype(phase)::value;
+        auto stage_of = [&](int off) __attribute__((always_inline)) -> int {
+            if constexpr (J >= 0) return (J + off) & (NST - 1);
+            else return (b + off) & (NST - 1);
+        };
+        if constexpr (J >= 0) {
+            // the fragment addresses are "redefined" here so that address + constant is formed
+            // inside the step (and folded into the read's immediate) instead of being hoisted
+            // out of the loop into one register per stage and fragment
+#pragma unroll
+            for (int i = 0; i < 8; i++) pin(kfo[i]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) pin(vfo[i]);
+        }
         auto mfma_slot = [&](int slot) __attribute__((always_inline)) {
             if (MFMA_PRIO) __builtin_amdgcn_s_setprio(MFMA_PRIO);
             if (slot & 1) {
@@ -567,7 +595,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 
         if constexpr (!XSTEP) {
 #pragma unroll
-            for (int g = 0; g < LA; g++) frag_read(b, g);
+            for (int g = 0; g < LA; g++) frag_read(stage_of(1), stage_of(NST - 1), g);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -577,8 +605,8 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
                 for (int j = 0; j < RB; j++) {
                     const int slot = g + LA + j;
-                    if (slot < 16) frag_read(b, slot);
-                    else if constexpr (XSTEP) frag_read(b + 1, slot - 16);
+                    if (slot < 16) frag_read(stage_of(1), stage_of(NST - 1), slot);
+                    else if constexpr (XSTEP) frag_read(stage_of(2), stage_of(0), slot - 16);
                 }
             }
             mfma_slot(g);
@@ -590,9 +618,9 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 if (g == 10) badm_cur = bmask[block_of(b + 1 < nblk ? b + 1 : nblk - 1)];
             }
             if constexpr (DMA) {
-                if (g == STORE_SLOT) dma_fetch(b + AHEAD);
+                if (g == STORE_SLOT) dma_fetch(b + AHEAD, stage_of(AHEAD));
             } else {
-                if (g == STORE_SLOT) stage_store(regs, (b + AHEAD) & (NST - 1));
+                if (g == STORE_SLOT) stage_store(regs, stage_of(AHEAD));
                 if (g == STORE_SLOT + 1) stage_load(regs, b + AHEAD + 2);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -629,7 +657,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         // prologue: blocks 0 .. AHEAD-1 into the ring, blocks AHEAD and AHEAD+1 in flight
         if constexpr (DMA) {
 #pragma unroll
-            for (int i = 0; i < AHEAD; i++) dma_fetch(i);
+            for (int i = 0; i < AHEAD; i++) dma_fetch(i, i);
             __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
         } else {
             StageRegs pre[AHEAD];
@@ -654,18 +682,33 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         qk_block(0, s_a);
         if constexpr (XSTEP) {
 #pragma unroll
-            for (int g = 0; g < LA; g++) frag_read(0, g);
+            for (int g = 0; g < LA; g++) frag_read(1, NST - 1, g);
         }
 
-        // two steps per trip so the S and P buffers swap roles without copies; with the
-        // 8-stage ring only the second step of a trip ends in a barrier
+        // Steps alternate the roles of the S and P buffers; with the 8-stage ring only odd
+        // steps end in a barrier. The main loop takes one full turn of the ring per trip
+        // with the ring phase a constant in every step; the remainder runs step by step.
+        typedef std::integral_constant<int, -1> Dyn;
         int b = 0;
+        // (builds that prepare K inside the block load carry too much state for a full turn)
+        for (; KMODE == kQkNone && b + NST <= nblk; b += NST) {
+            step(std::integral_constant<int, 0>{}, b, sets[0], NST != 8, s_a, s_b, p_a, p_b);
+            step(std::integral_constant<int, 1>{}, b + 1, sets[1], true, s_b, s_a, p_b, p_a);
+            step(std::integral_constant<int, 2>{}, b + 2, sets[0], NST != 8, s_a, s_b, p_a, p_b);
+            step(std::integral_constant<int, 3>{}, b + 3, sets[1], true, s_b, s_a, p_b, p_a);
+            if constexpr (NST == 8) {
+                step(std::integral_constant<int, 4>{}, b + 4, sets[0], false, s_a, s_b, p_a, p_b);
+                step(std::integral_constant<int, 5>{}, b + 5, sets[1], true, s_b, s_a, p_b, p_a);
+                step(std::integral_constant<int, 6>{}, b + 6, sets[0], false, s_a, s_b, p_a, p_b);
+                step(std::integral_constant<int, 7>{}, b + 7, sets[1], true, s_b, s_a, p_b, p_a);
+            }
+        }
         for (; b + 1 < nblk; b += 2) {
-            step(b, sets[0], NST != 8, s_a, s_b, p_a, p_b);
-            step(b + 1, sets[1], true, s_b, s_a, p_b, p_a);
+            step(Dyn{}, b, sets[0], NST != 8, s_a, s_b, p_a, p_b);
+            step(Dyn{}, b + 1, sets[1], true, s_b, s_a, p_b, p_a);
         }
         if (b < nblk) {
-            step(b, sets[0], true, s_a, s_b, p_a, p_b);
+            step(Dyn{}, b, sets[0], true, s_a, s_b, p_a, p_b);
             pv_block((nblk - 1) & (NST - 1), p_b);
         } else {
             pv_block((nblk - 1) & (NST - 1), p_a);
