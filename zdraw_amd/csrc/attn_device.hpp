@@ -198,10 +198,9 @@ __device__ __forceinline__ Rope8 ld_rope8(const QkOps& a, int mode, const QkRow&
     return t;
 }
 
-// x[0..7] (elements d0..d0+7 of a row) -> normalised, weighted, rotated.
-__device__ __forceinline__ void qk_apply8(int mode, float (&x)[8], float inv, const float* w, int d0, const Rope8& t) {
-    const f32x4 w0 = *reinterpret_cast<const f32x4*>(w + d0);
-    const f32x4 w1 = *reinterpret_cast<const f32x4*>(w + d0 + 4);
+// x[0..7] (elements d0..d0+7 of a row) -> normalised, weighted (w0, w1 = the 8 norm
+// weights of these elements), rotated.
+__device__ __forceinline__ void qk_apply8(int mode, float (&x)[8], float inv, const f32x4& w0, const f32x4& w1, const Rope8& t) {
     float y[8];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -226,6 +225,12 @@ __device__ __forceinline__ void qk_apply8(int mode, float (&x)[8], float inv, co
             x[2 * i + 1] = y[2 * i + 1] * c[i] + y[2 * i] * s[i];
         }
     }
+}
+// The same with the weights read from memory at w + d0.
+__device__ __forceinline__ void qk_apply8(int mode, float (&x)[8], float inv, const float* w, int d0, const Rope8& t) {
+    const f32x4 w0 = *reinterpret_cast<const f32x4*>(w + d0);
+    const f32x4 w1 = *reinterpret_cast<const f32x4*>(w + d0 + 4);
+    qk_apply8(mode, x, inv, w0, w1, t);
 }
 
 // Sum across the TPK adjacent lanes that share one K row (TPK = 4, 8 or 16).

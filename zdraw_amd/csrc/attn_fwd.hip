@@ -201,28 +201,48 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     bf16x8 qf[QB][8];
 #pragma unroll
     for (int qi = 0; qi < QB; qi++) {
-        const int qrow = q0 + 32 * qi + l32;
-        const bool ok = qrow < a.tokens;
-        const TIn* qp = reinterpret_cast<const TIn*>(a.q) + (int64_t)seg * a.q_bs + (int64_t)(ok ? qrow : 0) * a.q_ts +
+        // Rows past the sequence work on the last row (their output is never stored). All
+        // loads are unconditional and issued up front: a predicated load is a branch, and
+        // every branch here would wait for the loads before it.
+        const int qrow_raw = q0 + 32 * qi + l32;
+        const int qrow = qrow_raw < a.tokens ? qrow_raw : a.tokens - 1;
+        const TIn* qp = reinterpret_cast<const TIn*>(a.q) + (int64_t)seg * a.q_bs + (int64_t)qrow * a.q_ts +
                         (int64_t)head * a.q_hs + 8 * h;
-        float x[8][8];
+        Raw8<TIn> rawq[8];
 #pragma unroll
-        for (int s = 0; s < 8; s++) unpack8(ld_raw8<TIn>(qp + 16 * s, ok), x[s]);
+        for (int s = 0; s < 8; s++) rawq[s] = ld_raw8<TIn>(qp + 16 * s, true);
+        float x[8][8];
         if (a.q_mode != kQkNone) {
+            const QkRow r = qk_row(a.qk, a.q_mode, a.q_w, a.q_w_txt, seg, qrow, true);
+            Rope8 rope[4];
+            f32x4 w0[4], w1[4];
+            auto fetch_half = [&](int half) __attribute__((always_inline)) {
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    const int d0 = 16 * (4 * half + s) + 8 * h;
+                    rope[s] = ld_rope8(a.qk, a.q_mode, r, d0);
+                    w0[s] = *reinterpret_cast<const f32x4*>(r.w + d0);
+                    w1[s] = *reinterpret_cast<const f32x4*>(r.w + d0 + 4);
+                }
+            };
+            fetch_half(0);
             float ss = 0.f;
 #pragma unroll
-            for (int s = 0; s < 8; s++)
+            for (int s = 0; s < 8; s++) {
+                unpack8(rawq[s], x[s]);
 #pragma unroll
                 for (int i = 0; i < 8; i++) ss += x[s][i] * x[s][i];
+            }
             ss = pair_sum(ss);
             const float inv = rsqrtf(ss * (1.0f / D) + a.qk.eps);
-            const QkRow r = qk_row(a.qk, a.q_mode, a.q_w, a.q_w_txt, seg, qrow, ok);
 #pragma unroll
-            for (int s = 0; s < 8; s++) {
-                const int d0 = 16 * s + 8 * h;
-                const Rope8 t = ld_rope8(a.qk, a.q_mode, r, d0);
-                qk_apply8(a.q_mode, x[s], inv, r.w, d0, t);
-            }
+            for (int s = 0; s < 4; s++) qk_apply8(a.q_mode, x[s], inv, w0[s], w1[s], rope[s]);
+            fetch_half(1);
+#pragma unroll
+            for (int s = 0; s < 4; s++) qk_apply8(a.q_mode, x[4 + s], inv, w0[s], w1[s], rope[s]);
+        } else {
+#pragma unroll
+            for (int s = 0; s < 8; s++) unpack8(rawq[s], x[s]);
         }
         // log2(e)/sqrt(D) rides on Q, so the MFMA delivers scores in the exp2 domain
 #pragma unroll

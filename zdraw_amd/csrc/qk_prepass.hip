@@ -20,24 +20,30 @@ namespace zdraw {
 constexpr int kPrepTokens = 4; // tokens (waves) per workgroup
 constexpr int kPrepGroups = 6; // groups of four heads walked by one lane
 
-template <typename TIn>
+template <typename TIn, int MODE>
 __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const PrepArgs p) {
     constexpr int G = kPrepGroups;
     const int tok_raw = (int)blockIdx.x * kPrepTokens + (int)(threadIdx.x >> 6);
     const bool tok_ok = tok_raw < p.tokens;
-    const int tok = tok_ok ? tok_raw : 0;
+    const int tok = tok_ok ? tok_raw : p.tokens - 1; // lanes past the end work on the last token and store nothing
     const int h0 = (int)blockIdx.y * (4 * G) + (int)((threadIdx.x >> 4) & 3);
     const int seg = (int)blockIdx.z;
     const int d0 = (threadIdx.x & 15) * 8;
+    // Every load of the lane is issued before the first is used, with clamped addresses
+    // instead of predicates: no branch, so nothing waits for an earlier load to come back
+    // before the next is sent.
     const TIn* src = reinterpret_cast<const TIn*>(p.x) + (int64_t)seg * p.x_bs + (int64_t)tok * p.x_ts + d0;
     Raw8<TIn> raw[G];
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int head = h0 + 4 * g;
-        raw[g] = ld_raw8<TIn>(src + (int64_t)(head < p.heads ? head : 0) * p.x_hs, tok_ok && head < p.heads);
+        raw[g] = ld_raw8<TIn>(src + (int64_t)(head < p.heads ? head : p.heads - 1) * p.x_hs, true);
     }
-    const QkRow qr = qk_row(p.qk, p.mode, p.w, p.w_txt, seg, tok, tok_ok);
-    const Rope8 t = ld_rope8(p.qk, p.mode, qr, d0);
+    const QkRow qr = qk_row(p.qk, MODE, p.w, p.w_txt, seg, tok, true);
+    const Rope8 t = ld_rope8(p.qk, MODE, qr, d0);
+    // the token's weights and rope row stay in registers across its heads
+    const f32x4 w0 = *reinterpret_cast<const f32x4*>(qr.w + d0);
+    const f32x4 w1 = *reinterpret_cast<const f32x4*>(qr.w + d0 + 4);
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int head = h0 + 4 * g;
@@ -48,7 +54,7 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
         for (int i = 0; i < 8; i++) ss += x[i] * x[i];
         ss = row_group_sum<16>(ss);
         const float inv = rsqrtf(ss * (1.0f / D) + p.qk.eps);
-        qk_apply8(p.mode, x, inv, qr.w, d0, t);
+        qk_apply8(MODE, x, inv, w0, w1, t);
         if (tok_ok && head < p.heads) {
             const int64_t off = (int64_t)seg * p.y_bs + (int64_t)tok * p.y_ts + (int64_t)head * p.y_hs + d0;
             if (p.out_dtype == kF32) {
@@ -67,12 +73,17 @@ hipError_t launch_qk_prepass(const PrepArgs& p, int in_dtype, hipStream_t stream
     const dim3 grid((unsigned)((p.tokens + kPrepTokens - 1) / kPrepTokens),
                     (unsigned)((p.heads + 4 * kPrepGroups - 1) / (4 * kPrepGroups)), (unsigned)p.batch);
     const dim3 block(kPrepTokens * 64);
-    if (in_dtype == kF32)
-        qk_prepass_kernel<float><<<grid, block, 0, stream>>>(p);
-    else if (in_dtype == kBF16)
-        qk_prepass_kernel<bf16_t><<<grid, block, 0, stream>>>(p);
-    else
+    const bool klein = p.mode == kQkKlein;
+    if (!klein && p.mode != kQkZimage) return hipErrorInvalidValue;
+    if (in_dtype == kF32) {
+        if (klein) qk_prepass_kernel<float, kQkKlein><<<grid, block, 0, stream>>>(p);
+        else qk_prepass_kernel<float, kQkZimage><<<grid, block, 0, stream>>>(p);
+    } else if (in_dtype == kBF16) {
+        if (klein) qk_prepass_kernel<bf16_t, kQkKlein><<<grid, block, 0, stream>>>(p);
+        else qk_prepass_kernel<bf16_t, kQkZimage><<<grid, block, 0, stream>>>(p);
+    } else {
         return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 
