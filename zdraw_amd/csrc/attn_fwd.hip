@@ -198,59 +198,66 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     auto block_of = [&](int i) -> int { return (MASKED && kp) ? __builtin_amdgcn_readfirstlane((int)blocks[i]) : i; };
 
     // ---- Q rows -> B-operand registers: qf[qi][s], lane: query 32*qi + l32, dims 16s + 8h .. +7
+    // The workgroup's query rows are prepared in the layout that coalesces: 16 lanes per
+    // row (8 dims each, a row's 256 bytes and its rope row are contiguous), NT / 16 rows per
+    // pass. Norm, rope and the softmax scale are applied there and the bf16 rows are parked
+    // in LDS (the ring is not in use yet; 272-byte pitch, conflict-free b128 reads), from
+    // where every lane then picks up the fragments of ITS query row. A lane fetching its
+    // own row from memory would touch one cache line per lane and instruction.
+    // log2(e)/sqrt(D) rides on Q, so the MFMA delivers scores in the exp2 domain.
     bf16x8 qf[QB][8];
+    {
+        constexpr int QPITCH = D + 8;
+        constexpr int RPP = NT / 16;      // rows per pass
+        constexpr int PASSES = BQ / RPP;  // 8 QB
+        constexpr int BATCH = 4;          // passes whose loads are in flight together
+        bf16_t* const Qs = Ks;            // BQ x QPITCH elements at the start of the (idle) ring
+        const int prr = tid >> 4;
+        const int pd0 = (tid & 15) * 8;
+        const TIn* const qbase = reinterpret_cast<const TIn*>(a.q) + (int64_t)seg * a.q_bs + (int64_t)head * a.q_hs + pd0;
 #pragma unroll
-    for (int qi = 0; qi < QB; qi++) {
-        // Rows past the sequence work on the last row (their output is never stored). All
-        // loads are unconditional and issued up front: a predicated load is a branch, and
-        // every branch here would wait for the loads before it.
-        const int qrow_raw = q0 + 32 * qi + l32;
-        const int qrow = qrow_raw < a.tokens ? qrow_raw : a.tokens - 1;
-        const TIn* qp = reinterpret_cast<const TIn*>(a.q) + (int64_t)seg * a.q_bs + (int64_t)qrow * a.q_ts +
-                        (int64_t)head * a.q_hs + 8 * h;
-        Raw8<TIn> rawq[8];
+        for (int p0 = 0; p0 < PASSES; p0 += BATCH) {
+            Raw8<TIn> raw[BATCH];
+            QkRow rows[BATCH];
+            Rope8 rope[BATCH];
+            f32x4 w0[BATCH], w1[BATCH];
 #pragma unroll
-        for (int s = 0; s < 8; s++) rawq[s] = ld_raw8<TIn>(qp + 16 * s, true);
-        float x[8][8];
-        if (a.q_mode != kQkNone) {
-            const QkRow r = qk_row(a.qk, a.q_mode, a.q_w, a.q_w_txt, seg, qrow, true);
-            Rope8 rope[4];
-            f32x4 w0[4], w1[4];
-            auto fetch_half = [&](int half) __attribute__((always_inline)) {
-#pragma unroll
-                for (int s = 0; s < 4; s++) {
-                    const int d0 = 16 * (4 * half + s) + 8 * h;
-                    rope[s] = ld_rope8(a.qk, a.q_mode, r, d0);
-                    w0[s] = *reinterpret_cast<const f32x4*>(r.w + d0);
-                    w1[s] = *reinterpret_cast<const f32x4*>(r.w + d0 + 4);
+            for (int j = 0; j < BATCH; j++) {
+                // rows past the sequence work on the last row (their output is never stored)
+                const int qrow_raw = qb * BQ + (p0 + j) * RPP + prr;
+                const int qrow = qrow_raw < a.tokens ? qrow_raw : a.tokens - 1;
+                raw[j] = ld_raw8<TIn>(qbase + (int64_t)qrow * a.q_ts, true);
+                if (a.q_mode != kQkNone) {
+                    rows[j] = qk_row(a.qk, a.q_mode, a.q_w, a.q_w_txt, seg, qrow, true);
+                    rope[j] = ld_rope8(a.qk, a.q_mode, rows[j], pd0);
+                    w0[j] = *reinterpret_cast<const f32x4*>(rows[j].w + pd0);
+                    w1[j] = *reinterpret_cast<const f32x4*>(rows[j].w + pd0 + 4);
                 }
-            };
-            fetch_half(0);
-            float ss = 0.f;
-#pragma unroll
-            for (int s = 0; s < 8; s++) {
-                unpack8(rawq[s], x[s]);
-#pragma unroll
-                for (int i = 0; i < 8; i++) ss += x[s][i] * x[s][i];
             }
-            ss = pair_sum(ss);
-            const float inv = rsqrtf(ss * (1.0f / D) + a.qk.eps);
 #pragma unroll
-            for (int s = 0; s < 4; s++) qk_apply8(a.q_mode, x[s], inv, w0[s], w1[s], rope[s]);
-            fetch_half(1);
+            for (int j = 0; j < BATCH; j++) {
+                float x[8];
+                unpack8(raw[j], x);
+                if (a.q_mode != kQkNone) {
+                    float ss = 0.f;
 #pragma unroll
-            for (int s = 0; s < 4; s++) qk_apply8(a.q_mode, x[4 + s], inv, w0[s], w1[s], rope[s]);
-        } else {
+                    for (int i = 0; i < 8; i++) ss += x[i] * x[i];
+                    ss = row_group_sum<16>(ss);
+                    const float inv = rsqrtf(ss * (1.0f / D) + a.qk.eps);
+                    qk_apply8(a.q_mode, x, inv, w0[j], w1[j], rope[j]);
+                }
 #pragma unroll
-            for (int s = 0; s < 8; s++) unpack8(rawq[s], x[s]);
+                for (int i = 0; i < 8; i++) x[i] *= a.scale_log2;
+                *reinterpret_cast<u32x4*>(Qs + ((p0 + j) * RPP + prr) * QPITCH + pd0) = pack_bf16x8(x);
+            }
         }
-        // log2(e)/sqrt(D) rides on Q, so the MFMA delivers scores in the exp2 domain
+        __syncthreads();
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
+        for (int qi = 0; qi < QB; qi++)
 #pragma unroll
-            for (int i = 0; i < 8; i++) x[s][i] *= a.scale_log2;
-            qf[qi][s] = __builtin_bit_cast(bf16x8, pack_bf16x8(x[s]));
-        }
+            for (int s = 0; s < 8; s++)
+                qf[qi][s] = *reinterpret_cast<const bf16x8*>(Qs + (wave * QR + 32 * qi + l32) * QPITCH + 16 * s + 8 * h);
+        __syncthreads(); // the ring may be filled from here on
     }
 
     // ---- block staging: thread t owns key t/TPK of the block, CPT chunks of 8 dims of K and of V

@@ -79,10 +79,14 @@ struct PrepArgs {
     int32_t tokens, heads, batch;
     int32_t mode;       // QkMode (never kQkNone)
     int32_t out_dtype;  // kF32 or kBF16
-    int32_t pad0;
+    float scale;        // multiplies the result (1 for K; log2(e)/sqrt(head_dim) when Q is prepared for attention)
     QkOps qk;
     const float* w;
     const float* w_txt;
+};
+
+struct PrepPair {
+    PrepArgs op[2];
 };
 
 // Kernel shape: 0 = 8 waves x 32 query rows (one workgroup per CU, 8-stage LDS
@@ -93,7 +97,8 @@ int attention_max_tokens();
 // Launch one attention forward. in_dtype is kF32 or kBF16; k_mode is the
 // QkMode applied to K rows inside the K-block load. Returns a hipError_t.
 hipError_t launch_attention(const AttnArgs& args, int in_dtype, int k_mode, int shape, hipStream_t stream);
-hipError_t launch_qk_prepass(const PrepArgs& args, int in_dtype, hipStream_t stream);
+// Normalise + rotate `count` (1 or 2) operands of equal shape in one launch.
+hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipStream_t stream);
 // One-time per-device setup (raises the dynamic LDS limit on every instantiation).
 hipError_t attention_setup();
 

@@ -166,7 +166,8 @@ struct FusedPlan {
     int in_dtype;
     int k_mode;
     bool prepass;
-    PrepArgs prep;
+    PrepArgs prep;   // K pre-pass
+    PrepArgs prep_q; // Q pre-pass (same launch condition)
 };
 
 // Shared validation + argument assembly. Returns 0 or an ABI return code.
@@ -283,20 +284,21 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     plan->k_mode = (int)x->qk_mode;
     plan->prepass = false;
     if (x->qk_mode != ZDRAW_HIP_QK_NONE && x->k_site == ZDRAW_HIP_K_PREPASS) {
-        // K is normalised and rotated once into scratch slot 1, head-major, in
-        // the activation dtype; the attention kernel then reads it as is.
+        // Q and K are normalised and rotated once into scratch slots 0 and 1, head-major,
+        // in the activation dtype; the attention kernel then reads them as they are. One
+        // pass over the rows reads a token's rope row once for all its heads; inside the
+        // attention kernel every (head, query block) workgroup would fetch its own copy.
+        // Q also takes the softmax scale (in the exp2 domain) here, before the rounding.
         const size_t es = elem_size(x->in_dtype);
         const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * es;
-        Buffer* s = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 1, bytes));
-        if (!s) {
+        Buffer* sq = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 0, bytes));
+        Buffer* sk = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 1, bytes));
+        if (!sq || !sk) {
             set_err("scratch allocation failed");
             return ZDRAW_HIP_ERR_HANDLE;
         }
         PrepArgs pr;
         memset(&pr, 0, sizeof(pr));
-        pr.x = a.k;
-        pr.y = s->ptr;
-        pr.x_bs = a.k_bs; pr.x_ts = a.k_ts; pr.x_hs = a.k_hs;
         pr.y_bs = (int64_t)p->heads * p->tokens * kHeadDim;
         pr.y_ts = kHeadDim;
         pr.y_hs = (int64_t)p->tokens * kHeadDim;
@@ -304,13 +306,29 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         pr.mode = (int32_t)x->qk_mode;
         pr.out_dtype = (int32_t)x->in_dtype;
         pr.qk = a.qk;
+        PrepArgs pq = pr;
+        pr.x = a.k;
+        pr.y = sk->ptr;
+        pr.x_bs = a.k_bs; pr.x_ts = a.k_ts; pr.x_hs = a.k_hs;
         pr.w = a.k_w;
         pr.w_txt = a.k_w_txt;
+        pr.scale = 1.0f;
+        pq.x = a.q;
+        pq.y = sq->ptr;
+        pq.x_bs = a.q_bs; pq.x_ts = a.q_ts; pq.x_hs = a.q_hs;
+        pq.w = a.q_w;
+        pq.w_txt = a.q_w_txt;
+        pq.scale = a.scale_log2;
         plan->prep = pr;
+        plan->prep_q = pq;
         plan->prepass = true;
         plan->k_mode = kQkNone;
-        plan->args.k = s->ptr;
+        plan->args.k = sk->ptr;
         plan->args.k_bs = pr.y_bs; plan->args.k_ts = pr.y_ts; plan->args.k_hs = pr.y_hs;
+        plan->args.q = sq->ptr;
+        plan->args.q_bs = pr.y_bs; plan->args.q_ts = pr.y_ts; plan->args.q_hs = pr.y_hs;
+        plan->args.q_mode = kQkNone;
+        plan->args.scale_log2 = 1.0f;
     }
     return ZDRAW_HIP_OK;
 }
@@ -325,7 +343,8 @@ int enqueue(const FusedPlan& plan, hipStream_t stream) {
         g_setup_done = true;
     }
     if (plan.prepass) {
-        hipError_t e = launch_qk_prepass(plan.prep, plan.in_dtype, stream);
+        const PrepArgs both[2] = {plan.prep_q, plan.prep};
+        hipError_t e = launch_qk_prepass(both, 2, plan.in_dtype, stream);
         if (e != hipSuccess) {
             set_err("qk pre-pass launch: %s", hipGetErrorString(e));
             return ZDRAW_HIP_ERR_HANDLE;
@@ -741,10 +760,11 @@ int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
         pr.tokens = a.tokens; pr.heads = a.heads; pr.batch = 1;
         pr.mode = (int32_t)x->qk_mode;
         pr.out_dtype = kF32;
+        pr.scale = 1.0f;
         pr.qk = a.qk;
         pr.w = which == 0 ? a.q_w : a.k_w;
         pr.w_txt = which == 0 ? a.q_w_txt : a.k_w_txt;
-        hipError_t e = launch_qk_prepass(pr, kF32, qu->stream);
+        hipError_t e = launch_qk_prepass(&pr, 1, kF32, qu->stream);
         if (e != hipSuccess) {
             set_err("qk_norm_rope launch: %s", hipGetErrorString(e));
             return ZDRAW_HIP_ERR_HANDLE;

@@ -2,7 +2,7 @@
 //
 // Replaces krms_rope / krms_rope_hm (klein/zflux2_glue_shader.zig:61-122) and
 // qk_norm_rope / qk_norm_rope_hm_f16 (metal/mqk_shader.zig:46-97,
-// metal_api.m:6215-6265): used as the optional K pre-pass of the fused
+// metal_api.m:6215-6265): used as the optional Q/K pre-pass of the fused
 // attention entry and as the in-place f32 form behind zdraw_hip_run_qk_norm_rope.
 #include "attn_device.hpp"
 
@@ -14,20 +14,23 @@ namespace zdraw {
 // and walk G such groups of heads, keeping the token's rope coefficients and
 // norm weights in registers, so the rope table is read once per token. All G
 // loads of a lane are issued before the first is used. Input and output are
-// addressed by strides, so the same kernel serves the bf16 K pre-pass and the
+// addressed by strides, so the same kernel serves the 16-bit Q/K pre-pass and the
 // in-place f32 token-major form. A lane reads and writes only its own 8
 // elements, so the output may alias the input.
 constexpr int kPrepTokens = 4; // tokens (waves) per workgroup
 constexpr int kPrepGroups = 6; // groups of four heads walked by one lane
 
 template <typename TIn, int MODE>
-__global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const PrepArgs p) {
+__global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const PrepPair pair) {
     constexpr int G = kPrepGroups;
+    // grid z = operand * batch + segment; the choice is uniform over the workgroup
+    const int op = (int)blockIdx.z >= pair.op[0].batch ? 1 : 0;
+    const PrepArgs& p = pair.op[op];
     const int tok_raw = (int)blockIdx.x * kPrepTokens + (int)(threadIdx.x >> 6);
     const bool tok_ok = tok_raw < p.tokens;
     const int tok = tok_ok ? tok_raw : p.tokens - 1; // lanes past the end work on the last token and store nothing
     const int h0 = (int)blockIdx.y * (4 * G) + (int)((threadIdx.x >> 4) & 3);
-    const int seg = (int)blockIdx.z;
+    const int seg = (int)blockIdx.z - op * pair.op[0].batch;
     const int d0 = (threadIdx.x & 15) * 8;
     // Every load of the lane is issued before the first is used, with clamped addresses
     // instead of predicates: no branch, so nothing waits for an earlier load to come back
@@ -55,6 +58,8 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
         ss = row_group_sum<16>(ss);
         const float inv = rsqrtf(ss * (1.0f / D) + p.qk.eps);
         qk_apply8(MODE, x, inv, w0, w1, t);
+#pragma unroll
+        for (int i = 0; i < 8; i++) x[i] *= p.scale;
         if (tok_ok && head < p.heads) {
             const int64_t off = (int64_t)seg * p.y_bs + (int64_t)tok * p.y_ts + (int64_t)head * p.y_hs + d0;
             if (p.out_dtype == kF32) {
@@ -68,19 +73,28 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
     }
 }
 
-hipError_t launch_qk_prepass(const PrepArgs& p, int in_dtype, hipStream_t stream) {
-    if (p.batch <= 0 || p.heads <= 0 || p.tokens <= 0 || p.batch > 65535) return hipErrorInvalidValue;
+// One launch covers `count` operands (1 or 2) of equal tokens/heads/batch/mode.
+hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipStream_t stream) {
+    if (count < 1 || count > 2) return hipErrorInvalidValue;
+    const PrepArgs& p = ops[0];
+    if (p.batch <= 0 || p.heads <= 0 || p.tokens <= 0 || p.batch * count > 65535) return hipErrorInvalidValue;
+    if (count == 2 && (ops[1].batch != p.batch || ops[1].heads != p.heads || ops[1].tokens != p.tokens ||
+                       ops[1].mode != p.mode || ops[1].out_dtype != p.out_dtype))
+        return hipErrorInvalidValue;
+    PrepPair pair;
+    pair.op[0] = ops[0];
+    pair.op[1] = ops[count - 1];
     const dim3 grid((unsigned)((p.tokens + kPrepTokens - 1) / kPrepTokens),
-                    (unsigned)((p.heads + 4 * kPrepGroups - 1) / (4 * kPrepGroups)), (unsigned)p.batch);
+                    (unsigned)((p.heads + 4 * kPrepGroups - 1) / (4 * kPrepGroups)), (unsigned)(p.batch * count));
     const dim3 block(kPrepTokens * 64);
     const bool klein = p.mode == kQkKlein;
     if (!klein && p.mode != kQkZimage) return hipErrorInvalidValue;
     if (in_dtype == kF32) {
-        if (klein) qk_prepass_kernel<float, kQkKlein><<<grid, block, 0, stream>>>(p);
-        else qk_prepass_kernel<float, kQkZimage><<<grid, block, 0, stream>>>(p);
+        if (klein) qk_prepass_kernel<float, kQkKlein><<<grid, block, 0, stream>>>(pair);
+        else qk_prepass_kernel<float, kQkZimage><<<grid, block, 0, stream>>>(pair);
     } else if (in_dtype == kBF16) {
-        if (klein) qk_prepass_kernel<bf16_t, kQkKlein><<<grid, block, 0, stream>>>(p);
-        else qk_prepass_kernel<bf16_t, kQkZimage><<<grid, block, 0, stream>>>(p);
+        if (klein) qk_prepass_kernel<bf16_t, kQkKlein><<<grid, block, 0, stream>>>(pair);
+        else qk_prepass_kernel<bf16_t, kQkZimage><<<grid, block, 0, stream>>>(pair);
     } else {
         return hipErrorInvalidValue;
     }
