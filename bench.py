@@ -177,9 +177,93 @@ def gemm_main(args):
     print(json.dumps(line), flush=True)
 
 
+def chain_main(args):
+    """`--path chain`: the attention segment of one Z-Image layer at the zimage_1024 shape
+    (4608 tokens, 30 heads, hidden 3840): q/k/v projections, QK-norm + rope pre-pass, attention,
+    output projection, bf16 activations and weights. FLOPs = 4 projections + attention."""
+    import numpy as np
+
+    from zdraw_amd import hip, host
+    from zdraw_amd import workloads as wl
+
+    L = hip.lib()
+    ctx = host.Context.init()
+    w = wl.by_name("zimage_1024", seed=0)
+    tokens, heads = w.tokens, w.heads
+    hidden = inner = heads * 128
+    rng = np.random.default_rng(0)
+    bits = lambda a: host.f32_to_bf16_bits(a)
+    x = rng.standard_normal((tokens, hidden), dtype=np.float32)
+    wall_w = rng.standard_normal((4, inner, hidden), dtype=np.float32) * np.float32(hidden ** -0.5)
+    nb, wb = ctx.buffer(bits(x)), ctx.buffer(bits(wall_w))
+    qb, kb, vb, mixb, ob = (ctx.buffer(nbytes=tokens * inner * 2) for _ in range(5))
+    ones = ctx.buffer(np.ones(128, np.float32))
+    posb = ctx.buffer(np.ascontiguousarray(w.pos, dtype=np.uint64))
+    ropeb = ctx.buffer(w.rope_pairs)
+    p = hip.ChainAttnParams()
+    for i, name in enumerate(("q", "k", "v", "proj")):
+        setattr(p, name, hip.GemmParams(tokens, hidden, inner, hip.W_BF16, hip.GEMM_HALF, i * inner * hidden * 2))
+    p.qk = hip.QkNormParams(tokens, heads, heads, 128, hip.W_F32, hip.W_F32, *wl.ZIMAGE_DIMS, wl.ZIMAGE_EPS, 0, 0,
+                            *w.rope_bases)
+    p.attn = hip.AttnParams(tokens, heads, heads, 128, 0, 0)
+    p.act_dtype = hip.BF16
+    p.score_bound = host.score_bound(np.ones(128, np.float32), np.ones(128, np.float32), None, None)
+    bufs = hip.ChainAttnBuffers(nb.handle, qb.handle, kb.handle, vb.handle, mixb.handle, ob.handle)
+    wts = hip.ChainAttnWeights(wb.handle, wb.handle, wb.handle, ones.handle, ones.handle, posb.handle, ropeb.handle,
+                               wb.handle)
+
+    def burst(count):
+        b = L.zdraw_hip_batch_begin(ctx.queue)
+        for _ in range(count):
+            rc = L.zdraw_hip_run_chain_attn_enc(b, C.byref(bufs), C.byref(wts), C.byref(p))
+            if rc != 0:
+                raise RuntimeError(f"chain rc={rc}: {hip.last_error()}")
+        if L.zdraw_hip_batch_end(b) != 0:
+            raise RuntimeError("batch_end failed")
+
+    t0 = time.perf_counter()
+    spun = 0
+    while (time.perf_counter() - t0) * 1e3 < args.spinup_ms:
+        burst(20)
+        spun += 20
+    burst(max(args.warmup, 1))
+    e0, e1 = L.zdraw_hip_event_create(), L.zdraw_hip_event_create()
+    L.zdraw_hip_queue_sync(ctx.queue)
+    t0 = time.perf_counter()
+    L.zdraw_hip_event_record(e0, ctx.queue)
+    burst(args.steps)
+    L.zdraw_hip_event_record(e1, ctx.queue)
+    L.zdraw_hip_event_sync(e1)
+    wall = time.perf_counter() - t0
+    dev_ms = L.zdraw_hip_event_elapsed_ms(e0, e1) / args.steps
+    out = host.bf16_bits_to_f32(ob.read(np.uint16, (tokens, hidden)))
+    if not np.isfinite(out).all():
+        raise RuntimeError("non-finite output")
+    gemm_flops = 4 * 2.0 * tokens * hidden * inner
+    attn_flops = 4.0 * 128 * heads * tokens * tokens
+    flops = gemm_flops + attn_flops
+    value = flops / (wall / args.steps) / 1e12
+    line = {
+        "metric": "Z-Image layer attention segment TFLOP/s (4 projections + attention)",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"zimage chain segment: tokens {tokens}, heads {heads}, hidden {hidden}, bf16 activations and weights",
+                   "gemm_gflop": gemm_flops / 1e9, "attention_gflop": attn_flops / 1e9,
+                   "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS, "untimed_spinup_segments": spun},
+        "roofline": {"bound": "mfma", "achieved": flops / (dev_ms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": flops / (dev_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "3 x gemm + qk_prepass + attn_fwd + gemm", "kernel_ms": dev_ms},
+    }
+    for b in (nb, wb, qb, kb, vb, mixb, ob, ones, posb, ropeb):
+        b.release()
+    ctx.deinit()
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--path", choices=["attention", "gemm"], default="attention",
+    ap.add_argument("--path", choices=["attention", "gemm", "chain"], default="attention",
                     help="attention (the headline metric) or the projection GEMM beside it")
     ap.add_argument("--m", type=int, default=4608)
     ap.add_argument("--k", type=int, default=3072)
@@ -204,6 +288,8 @@ def main():
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)")
     if args.path == "gemm":
         return gemm_main(args)
+    if args.path == "chain":
+        return chain_main(args)
 
     import numpy as np
 

@@ -63,10 +63,10 @@ enum {
     ZDRAW_HIP_QK_ZIMAGE = 2 /* qk_norm_rope: metal/mqk_shader.zig:46-97 */
 };
 
-/* Where K's norm+rope happens for the fused entry. */
+/* Where norm+rope happens for the fused entry. */
 enum {
-    ZDRAW_HIP_K_IN_TILE_LOAD = 0, /* inside the attention kernel, per K tile */
-    ZDRAW_HIP_K_PREPASS = 1       /* one pre-pass kernel into library scratch, then attention */
+    ZDRAW_HIP_K_IN_TILE_LOAD = 0, /* inside the attention kernel: Q in its prologue, K per tile */
+    ZDRAW_HIP_K_PREPASS = 1       /* one pre-pass kernel prepares Q and K into library scratch, then attention */
 };
 
 /*
@@ -221,11 +221,76 @@ int zdraw_hip_run_gemm_off_enc(void* batch, void* pipeline, void* a, void* w, vo
 /* metal_c.zig:425-433 (and :378-386): A already in the weight's 16-bit type, C f32. */
 int zdraw_hip_run_gemm_f16a_enc(void* batch, void* a, void* w, void* c, const ZdrawGemmParams* params,
                                 uint64_t a_offset, uint64_t c_offset);
+/* metal_c.zig:175-198: two or three products of the same A (f32 in, f32 out), blocking.
+ * Products of equal shape and weight type run as one launch whose tiles cover all
+ * of them; otherwise one launch each. */
+int zdraw_hip_run_gemm_pair(void* queue, void* pipeline, void* a, void* w0, void* c0, const ZdrawGemmParams* params0,
+                            void* w1, void* c1, const ZdrawGemmParams* params1);
+int zdraw_hip_run_gemm_triple(void* queue, void* pipeline, void* a, void* w0, void* c0, const ZdrawGemmParams* params0,
+                              void* w1, void* c1, const ZdrawGemmParams* params1, void* w2, void* c2,
+                              const ZdrawGemmParams* params2);
 /* General form: leading dimensions and 16-bit output, e.g. Q/K/V written as
  * bf16 token-major rows for the attention entry, or the attention output read
  * from the concat operand at its row pitch. */
 int zdraw_hip_run_gemm_ext_enc(void* batch, void* a, void* w, void* c, const ZdrawGemmParams* params,
                                const ZdrawHipGemmExt* ext);
+
+/* ---- Z-Image layer, attention segment --------------------------------------
+ * The q/k/v projections, QK-norm + rope, attention and output projection of one
+ * Z-Image layer as metal_api.m:7134-7212 (encode_chain_layer_ours16) and
+ * :7103-7108 (encode_chain_layer) encode them:
+ *   q = norm x Wq^T, k = norm x Wk^T, v = norm x Wv^T      (GemmParams q, k, v)
+ *   qk_norm_rope(q, k; q_norm, k_norm, pos, rope)           (QkNormParams qk)
+ *   mix = attention(q, k, v)                                (AttnParams attn)
+ *   attn = mix x Wproj^T                                    (GemmParams proj)
+ * The structs carry the fields of ZdrawBlockBuffers / ZdrawBlockWeights /
+ * ZdrawBlockChainParams (metal_api.m:5961-5987) that this segment reads, in the
+ * reference's order. Rows padded to a multiple of 32 (zimage/zseq.zig:23-34) are
+ * ordinary rows here, as they are there. */
+typedef struct ZdrawQkNormParams { /* metal_c.zig:258-274, 80 bytes */
+    uint32_t tokens, heads, kv_heads, head_dim;
+    uint32_t q_dtype, k_dtype; /* element type of q_norm / k_norm: 1 f16, 2 bf16, 3 f32 */
+    uint32_t dim0, dim1, dim2; /* rope axis widths, sum = head_dim */
+    float eps;
+    uint64_t q_offset, k_offset; /* byte offsets of the norm weights in their buffers */
+    uint64_t base0, base1, base2; /* axis bases in (cos,sin) pairs */
+} ZdrawQkNormParams;
+
+typedef struct ZdrawHipChainAttnBuffers {
+    void* norm; /* [tokens][hidden] layer input after its norm (activation dtype) */
+    void* q;    /* [tokens][heads*128]; holds the raw projection afterwards */
+    void* k;
+    void* v;
+    void* mix;  /* [tokens][heads*128] attention output */
+    void* attn; /* [tokens][hidden] projected output */
+} ZdrawHipChainAttnBuffers;
+
+typedef struct ZdrawHipChainAttnWeights {
+    void* q; void* k; void* v; /* [heads*128][hidden], 16-bit */
+    void* q_norm; void* k_norm; /* [128] */
+    void* pos;  /* u64 [tokens][3] */
+    void* rope; /* (cos,sin) f32 pairs */
+    void* proj; /* [hidden][heads*128], 16-bit */
+} ZdrawHipChainAttnWeights;
+
+typedef struct ZdrawHipChainAttnParams {
+    ZdrawGemmParams q, k, v;
+    ZdrawQkNormParams qk;
+    ZdrawAttnParams attn;
+    ZdrawGemmParams proj;
+    /* no counterpart in the reference (its chain buffers are f32): element type of
+     * every buffer in ZdrawHipChainAttnBuffers, ZDRAW_HIP_F32 or ZDRAW_HIP_BF16
+     * (the latter needs bf16 weights). */
+    uint32_t act_dtype;
+    float score_bound; /* as ZdrawHipAttnExt.score_bound; 0 = unknown */
+} ZdrawHipChainAttnParams;
+
+/* Enqueues the launches (q/k/v projections as one, pre-pass, attention, projection) on the batch's stream. 0 = enqueued; 1 = a shape or
+ * weight form this backend does not run (nothing enqueued, the caller keeps its
+ * own path); negative = invalid arguments. */
+int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* buffers,
+                                 const ZdrawHipChainAttnWeights* weights,
+                                 const ZdrawHipChainAttnParams* params);
 
 /* ---- library-owned scratch (metal_c.zig:321-325) -------------------------- */
 /* Grow-only, process-lifetime, filled at (re)allocation with 0x00 (0xFF when
@@ -279,7 +344,8 @@ void zdraw_hip_set_attention_variant(int variant);
 /* ABI drift guard (src/abi_gen.zig, runtime/abi_assert.zig:29): sizeof of the
  * shared structs as this library was compiled. which: 0 = ZdrawAttnParams,
  * 1 = ZdrawHipAttnExt, 2 = ZdrawHipQkOperands, 3 = ZdrawGemmParams,
- * 4 = ZdrawHipGemmExt. */
+ * 4 = ZdrawHipGemmExt, 5 = ZdrawQkNormParams, 6 = ZdrawHipChainAttnBuffers,
+ * 7 = ZdrawHipChainAttnWeights, 8 = ZdrawHipChainAttnParams. */
 size_t zdraw_hip_abi_sizeof(int which);
 /* Last error text of this thread's most recent failing call ("" if none). */
 const char* zdraw_hip_last_error(void);
@@ -289,6 +355,10 @@ const char* zdraw_hip_last_error(void);
 #define ZDRAW_HIP_ABI_QK_OPERANDS_SIZE 72
 #define ZDRAW_HIP_ABI_GEMM_PARAMS_SIZE 32
 #define ZDRAW_HIP_ABI_GEMM_EXT_SIZE 48
+#define ZDRAW_HIP_ABI_QK_NORM_PARAMS_SIZE 80
+#define ZDRAW_HIP_ABI_CHAIN_ATTN_BUFFERS_SIZE 48
+#define ZDRAW_HIP_ABI_CHAIN_ATTN_WEIGHTS_SIZE 64
+#define ZDRAW_HIP_ABI_CHAIN_ATTN_PARAMS_SIZE 240
 
 #ifdef __cplusplus
 }

@@ -40,7 +40,18 @@ def test_abi_struct_sizes():
     assert L.zdraw_hip_abi_sizeof(3) == C.sizeof(hip.GemmParams) == 32
     assert hip.GemmParams.weight_offset.offset == 24
     assert L.zdraw_hip_abi_sizeof(4) == C.sizeof(hip.GemmExt) == 48
+    # QkNormParams keeps the reference's 80 bytes (metal_c.zig:258-274); in the chain
+    # parameters qk follows three GemmParams and proj sits 104 bytes after qk, as in
+    # ZdrawBlockChainParams (metal_api.m:6007-6008: qk at 128, proj at 232)
+    assert L.zdraw_hip_abi_sizeof(5) == C.sizeof(hip.QkNormParams) == 80
+    assert hip.QkNormParams.q_offset.offset == 40 and hip.QkNormParams.base0.offset == 56
+    assert L.zdraw_hip_abi_sizeof(6) == C.sizeof(hip.ChainAttnBuffers) == 48
+    assert L.zdraw_hip_abi_sizeof(7) == C.sizeof(hip.ChainAttnWeights) == 64
+    assert L.zdraw_hip_abi_sizeof(8) == C.sizeof(hip.ChainAttnParams) == 240
+    assert hip.ChainAttnParams.proj.offset - hip.ChainAttnParams.qk.offset == 232 - 128
     text = open(os.path.join(ROOT, "include", "zdraw_hip.h")).read()
+    assert "#define ZDRAW_HIP_ABI_QK_NORM_PARAMS_SIZE 80" in text
+    assert "#define ZDRAW_HIP_ABI_CHAIN_ATTN_PARAMS_SIZE 240" in text
     assert "#define ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE 24" in text
     assert "#define ZDRAW_HIP_ABI_ATTN_EXT_SIZE 216" in text
     assert "#define ZDRAW_HIP_ABI_QK_OPERANDS_SIZE 72" in text

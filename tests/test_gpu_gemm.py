@@ -263,3 +263,51 @@ def test_single_block_chain_projection_attention_projection(ctx):
     assert err.max() <= 2e-2 * max(s, 1.0) and err.mean() <= 2e-3 * max(s, 1.0), (err.max(), err.mean(), s)
     for b in [xb, wqkvb, woutb, cat, out, nqb, nkb, cos, sin] + qkv:
         b.release()
+
+
+@pytest.mark.parametrize("count", [2, 3])
+@pytest.mark.parametrize("same_shape", [True, False])
+def test_pair_and_triple_of_one_activation(ctx, pipe, count, same_shape):
+    # metal_c.zig:175-198: gate/up (pair) and q/k/v (triple) products of one f32 A, blocking.
+    # Equal shapes run as ONE launch, unequal ones as one launch each; results are those of
+    # `count` separate zdraw_hip_run_gemm calls, bit for bit.
+    L = hip.lib()
+    rng = np.random.default_rng(17 + count)
+    m, k = 300, 136
+    ns = [264] * count if same_shape else [264, 128, 40][:count]
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    ws = [rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5) for n in ns]
+    # all weights in one buffer behind a 32-byte header: weight_offset selects them
+    bits = [to16(w, hip.W_F16)[0] for w in ws]
+    blob = np.concatenate([np.zeros(16, np.uint16)] + [b.ravel() for b in bits])
+    offs = [32 + 2 * sum(n * k for n in ns[:i]) for i in range(count)]
+    ab, wb = ctx.buffer(a), ctx.buffer(blob)
+    cbs = [ctx.buffer(nbytes=m * n * 4) for n in ns]
+    ps = [hip.GemmParams(m, k, n, hip.W_F16, hip.GEMM_HALF, off) for n, off in zip(ns, offs)]
+    d0 = L.zdraw_hip_dispatch_count()
+    if count == 2:
+        rc = L.zdraw_hip_run_gemm_pair(ctx.queue, pipe, ab.handle, wb.handle, cbs[0].handle, C.byref(ps[0]),
+                                       wb.handle, cbs[1].handle, C.byref(ps[1]))
+    else:
+        rc = L.zdraw_hip_run_gemm_triple(ctx.queue, pipe, ab.handle, wb.handle, cbs[0].handle, C.byref(ps[0]),
+                                         wb.handle, cbs[1].handle, C.byref(ps[1]), wb.handle, cbs[2].handle, C.byref(ps[2]))
+    assert rc == 0, hip.last_error()
+    assert L.zdraw_hip_dispatch_count() - d0 == (1 if same_shape else count)
+    ar = to16(a, hip.W_F16)[1]
+    for i, n in enumerate(ns):
+        got = cbs[i].read(np.float32, (m, n))
+        wr = from16(bits[i], hip.W_F16)
+        check(got, zo.linear_batch(ar, wr), zo.linear_batch(a, ws[i]), k, a, ws[i], f"product {i} of {count}")
+        single = ctx.buffer(nbytes=m * n * 4)
+        assert L.zdraw_hip_run_gemm(ctx.queue, pipe, ab.handle, wb.handle, single.handle, C.byref(ps[i])) == 0
+        assert np.array_equal(single.read(np.float32, (m, n)), got)
+        single.release()
+    # a product this backend does not run refuses the whole call before anything is enqueued
+    bad = hip.GemmParams(m, k, ns[-1], hip.W_F32, hip.GEMM_HALF, 0)
+    d0 = L.zdraw_hip_dispatch_count()
+    if count == 2 and not same_shape:
+        assert L.zdraw_hip_run_gemm_pair(ctx.queue, pipe, ab.handle, wb.handle, cbs[0].handle, C.byref(ps[0]),
+                                         wb.handle, cbs[1].handle, C.byref(bad)) == 1
+        assert L.zdraw_hip_dispatch_count() == d0
+    for b in [ab, wb] + cbs:
+        b.release()

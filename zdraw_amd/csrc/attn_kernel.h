@@ -81,8 +81,10 @@ struct PrepArgs {
     int32_t out_dtype;  // kF32 or kBF16
     float scale;        // multiplies the result (1 for K; log2(e)/sqrt(head_dim) when Q is prepared for attention)
     QkOps qk;
-    const float* w;
-    const float* w_txt;
+    const void* w;      // 128 norm weights, element type w_dtype
+    const void* w_txt;
+    int32_t w_dtype;    // kF32, kF16 or kBF16
+    int32_t pad0;
 };
 
 struct PrepPair {

@@ -27,6 +27,10 @@ static_assert(sizeof(ZdrawHipAttnExt) == ZDRAW_HIP_ABI_ATTN_EXT_SIZE, "AttnExt A
 static_assert(sizeof(ZdrawHipQkOperands) == ZDRAW_HIP_ABI_QK_OPERANDS_SIZE, "QkOperands ABI drift");
 static_assert(sizeof(ZdrawGemmParams) == ZDRAW_HIP_ABI_GEMM_PARAMS_SIZE, "GemmParams ABI drift");
 static_assert(sizeof(ZdrawHipGemmExt) == ZDRAW_HIP_ABI_GEMM_EXT_SIZE, "GemmExt ABI drift");
+static_assert(sizeof(ZdrawQkNormParams) == ZDRAW_HIP_ABI_QK_NORM_PARAMS_SIZE, "QkNormParams ABI drift");
+static_assert(sizeof(ZdrawHipChainAttnBuffers) == ZDRAW_HIP_ABI_CHAIN_ATTN_BUFFERS_SIZE, "ChainAttnBuffers ABI drift");
+static_assert(sizeof(ZdrawHipChainAttnWeights) == ZDRAW_HIP_ABI_CHAIN_ATTN_WEIGHTS_SIZE, "ChainAttnWeights ABI drift");
+static_assert(sizeof(ZdrawHipChainAttnParams) == ZDRAW_HIP_ABI_CHAIN_ATTN_PARAMS_SIZE, "ChainAttnParams ABI drift");
 
 namespace {
 
@@ -168,11 +172,25 @@ struct FusedPlan {
     bool prepass;
     PrepArgs prep;   // K pre-pass
     PrepArgs prep_q; // Q pre-pass (same launch condition)
+    int w_dtype = kF32; // element type of the norm weights (16-bit only with the pre-pass)
 };
 
+// Norm weights as QkNormParams describes them (metal_c.zig:258-274): element
+// type in the weight coding (1 f16, 2 bf16, 3 f32) and a byte offset into the buffer.
+struct NormWeights {
+    uint32_t q_dtype, k_dtype;
+    uint64_t q_off, k_off;
+};
+
+int norm_weight_dtype(uint32_t coded) {
+    return coded == ZDRAW_HIP_W_F32 ? (int)kF32 : coded == ZDRAW_HIP_W_F16 ? (int)kF16 : coded == ZDRAW_HIP_W_BF16 ? (int)kBF16 : -1;
+}
+
 // Shared validation + argument assembly. Returns 0 or an ABI return code.
+// nw == nullptr: norm weights are f32[128] at offset 0.
 int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const ZdrawAttnParams* p,
-                   const ZdrawHipAttnExt* x, const ZdrawHipQkOperands* ops, FusedPlan* plan) {
+                   const ZdrawHipAttnExt* x, const ZdrawHipQkOperands* ops, FusedPlan* plan,
+                   const NormWeights* nw = nullptr) {
     if (!p || !x) {
         set_err("null params");
         return ZDRAW_HIP_ERR_HANDLE;
@@ -230,14 +248,31 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     const uint64_t rows_needed = (uint64_t)(x->batch - 1) * x->rope_batch_rows + p->tokens;
     if (x->qk_mode != ZDRAW_HIP_QK_NONE) {
         if (!ops) return invalid("qk_mode set without operands");
-        if (!need(ops->q_weight, kHeadDim * 4) || !need(ops->k_weight, kHeadDim * 4))
-            return invalid("norm weights must be f32[128] buffers");
+        int qwd = kF32, kwd = kF32;
+        uint64_t qwo = 0, kwo = 0;
+        if (nw) {
+            qwd = norm_weight_dtype(nw->q_dtype);
+            kwd = norm_weight_dtype(nw->k_dtype);
+            qwo = nw->q_off;
+            kwo = nw->k_off;
+            if (qwd < 0 || kwd < 0 || qwd != kwd) return unavailable("norm weight dtype");
+            if (qwd != kF32 && x->k_site != ZDRAW_HIP_K_PREPASS) return unavailable("16-bit norm weights need the pre-pass");
+            if (qwo % 16 != 0 || kwo % 16 != 0) return invalid("norm weight offsets must be 16-byte aligned");
+            if (ops->q_weight_txt || ops->k_weight_txt) return invalid("text norm weights with typed norm weights");
+        }
+        const size_t wbytes = (size_t)kHeadDim * (qwd == kF32 ? 4 : 2);
+        if (!ops->q_weight || !ops->k_weight || qwo > static_cast<Buffer*>(ops->q_weight)->len ||
+            kwo > static_cast<Buffer*>(ops->k_weight)->len ||
+            static_cast<Buffer*>(ops->q_weight)->len - qwo < wbytes || static_cast<Buffer*>(ops->k_weight)->len - kwo < wbytes ||
+            !static_cast<Buffer*>(ops->q_weight)->ptr || !static_cast<Buffer*>(ops->k_weight)->ptr)
+            return invalid("norm weights must be [128] buffers (f32 unless the caller states a type)");
+        plan->w_dtype = qwd;
         if ((ops->q_weight_txt && !need(ops->q_weight_txt, kHeadDim * 4)) ||
             (ops->k_weight_txt && !need(ops->k_weight_txt, kHeadDim * 4)))
             return invalid("text norm weights must be f32[128] buffers");
         if (!(x->eps >= 0.0f)) return invalid("eps");
-        a.q_w = static_cast<const float*>(static_cast<Buffer*>(ops->q_weight)->ptr);
-        a.k_w = static_cast<const float*>(static_cast<Buffer*>(ops->k_weight)->ptr);
+        a.q_w = reinterpret_cast<const float*>(static_cast<const char*>(static_cast<Buffer*>(ops->q_weight)->ptr) + qwo);
+        a.k_w = reinterpret_cast<const float*>(static_cast<const char*>(static_cast<Buffer*>(ops->k_weight)->ptr) + kwo);
         a.q_w_txt = ops->q_weight_txt ? static_cast<const float*>(static_cast<Buffer*>(ops->q_weight_txt)->ptr) : nullptr;
         a.k_w_txt = ops->k_weight_txt ? static_cast<const float*>(static_cast<Buffer*>(ops->k_weight_txt)->ptr) : nullptr;
         a.qk.txt_rows = (int32_t)x->txt_rows;
@@ -306,6 +341,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         pr.mode = (int32_t)x->qk_mode;
         pr.out_dtype = (int32_t)x->in_dtype;
         pr.qk = a.qk;
+        pr.w_dtype = plan->w_dtype;
         PrepArgs pq = pr;
         pr.x = a.k;
         pr.y = sk->ptr;
@@ -434,8 +470,11 @@ bool scratch_poisoned(int slot) {
 }
 
 // C = A x W^T (metal_api.m gemm encode paths). Validates, then launches on `stream`.
-int enqueue_gemm(void* a, void* w, void* c, const ZdrawGemmParams* p, const ZdrawHipGemmExt* x, hipStream_t stream) {
-    if (!p || !x) {
+// One launch for `groups` (1..3) products that share A, every dimension and the
+// extension block: group i multiplies by ws[i] at byte offset w_offs[i] into cs[i].
+int enqueue_gemm_group(void* a, void* const* ws, void* const* cs, const uint64_t* w_offs, int groups,
+                       const ZdrawGemmParams* p, const ZdrawHipGemmExt* x, hipStream_t stream) {
+    if (!p || !x || groups < 1 || groups > 3) {
         set_err("null params");
         return ZDRAW_HIP_ERR_HANDLE;
     }
@@ -447,24 +486,27 @@ int enqueue_gemm(void* a, void* w, void* c, const ZdrawGemmParams* p, const Zdra
     if ((x->a_dtype != ZDRAW_HIP_F32 && x->a_dtype != wt) || (x->c_dtype != ZDRAW_HIP_F32 && x->c_dtype != wt))
         return invalid("activation / output dtype must be f32 or the weight's type");
     const Buffer* ab = static_cast<const Buffer*>(a);
-    const Buffer* wb = static_cast<const Buffer*>(w);
-    const Buffer* cb = static_cast<const Buffer*>(c);
-    if (!ab || !wb || !cb || !ab->ptr || !wb->ptr || !cb->ptr) return invalid("null buffer");
+    if (!ab || !ab->ptr) return invalid("null buffer");
     const uint64_t lda = x->lda ? x->lda : p->k, ldw = x->ldw ? x->ldw : p->k, ldc = x->ldc ? x->ldc : p->n;
     if (lda < p->k || ldw < p->k || ldc < p->n) return invalid("leading dimension smaller than the row");
     const uint64_t ea = elem_size(x->a_dtype), ec = elem_size(x->c_dtype);
     // 16-byte loads of 8 (16-bit) or 4 (f32) elements: rows must start 16-byte aligned
     if (x->a_off % 16 != 0 || (lda * ea) % 16 != 0 || ((uintptr_t)ab->ptr % 16) != 0) return invalid("A rows not 16-byte aligned");
-    if (p->weight_offset % 16 != 0 || (ldw * 2) % 16 != 0 || ((uintptr_t)wb->ptr % 16) != 0) return invalid("W rows not 16-byte aligned");
     if (x->c_off % ec != 0) return invalid("C offset not element aligned");
     const uint64_t a_bytes = ((uint64_t)(p->m - 1) * lda + p->k) * ea;
     const uint64_t w_bytes = ((uint64_t)(p->n - 1) * ldw + p->k) * 2;
     const uint64_t c_bytes = ((uint64_t)(p->m - 1) * ldc + p->n) * ec;
     if (x->a_off > ab->len || a_bytes > ab->len - x->a_off) return invalid("A buffer too small");
-    if (p->weight_offset > wb->len || w_bytes > wb->len - p->weight_offset) return invalid("W buffer too small");
-    if (x->c_off > cb->len || c_bytes > cb->len - x->c_off) return invalid("C buffer too small");
     // the kernel addresses A and W with 32-bit byte offsets from their first element
     if (a_bytes >= (1ull << 32) || w_bytes >= (1ull << 32)) return unavailable("operand spans 4 GiB or more");
+    for (int i = 0; i < groups; i++) {
+        const Buffer* wb = static_cast<const Buffer*>(ws[i]);
+        const Buffer* cb = static_cast<const Buffer*>(cs[i]);
+        if (!wb || !cb || !wb->ptr || !cb->ptr) return invalid("null buffer");
+        if (w_offs[i] % 16 != 0 || (ldw * 2) % 16 != 0 || ((uintptr_t)wb->ptr % 16) != 0) return invalid("W rows not 16-byte aligned");
+        if (w_offs[i] > wb->len || w_bytes > wb->len - w_offs[i]) return invalid("W buffer too small");
+        if (x->c_off > cb->len || c_bytes > cb->len - x->c_off) return invalid("C buffer too small");
+    }
     if (!g_gemm_setup_done) {
         hipError_t e = gemm_setup();
         if (e != hipSuccess) {
@@ -476,12 +518,17 @@ int enqueue_gemm(void* a, void* w, void* c, const ZdrawGemmParams* p, const Zdra
     GemmArgs g;
     memset(&g, 0, sizeof(g));
     g.a = static_cast<const char*>(ab->ptr) + x->a_off;
-    g.w = static_cast<const char*>(wb->ptr) + p->weight_offset;
-    g.c = static_cast<char*>(cb->ptr) + x->c_off;
+    g.w = static_cast<const char*>(static_cast<const Buffer*>(ws[0])->ptr) + w_offs[0];
+    g.c = static_cast<char*>(static_cast<const Buffer*>(cs[0])->ptr) + x->c_off;
+    g.groups = groups;
+    for (int i = 1; i < groups; i++) {
+        g.w_more[i - 1] = static_cast<const char*>(static_cast<const Buffer*>(ws[i])->ptr) + w_offs[i];
+        g.c_more[i - 1] = static_cast<char*>(static_cast<const Buffer*>(cs[i])->ptr) + x->c_off;
+    }
     g.m = (int32_t)p->m; g.n = (int32_t)p->n; g.k = (int32_t)p->k;
     g.lda = (int64_t)lda; g.ldw = (int64_t)ldw; g.ldc = (int64_t)ldc;
     g.tiles_n = (int32_t)((p->n + (uint32_t)gemm_tile_cols() - 1) / (uint32_t)gemm_tile_cols());
-    if ((uint64_t)g.tiles_n * ((p->m + (uint32_t)gemm_tile_rows() - 1) / (uint32_t)gemm_tile_rows()) > 0x7fffffffull)
+    if ((uint64_t)g.tiles_n * (uint64_t)groups * ((p->m + (uint32_t)gemm_tile_rows() - 1) / (uint32_t)gemm_tile_rows()) > 0x7fffffffull)
         return unavailable("grid too large");
     hipError_t e = launch_gemm(g, (int)x->a_dtype, (int)wt, (int)x->c_dtype, stream);
     if (e != hipSuccess) {
@@ -490,6 +537,14 @@ int enqueue_gemm(void* a, void* w, void* c, const ZdrawGemmParams* p, const Zdra
     }
     g_dispatch++;
     return ZDRAW_HIP_OK;
+}
+
+int enqueue_gemm(void* a, void* w, void* c, const ZdrawGemmParams* p, const ZdrawHipGemmExt* x, hipStream_t stream) {
+    if (!p) {
+        set_err("null params");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    return enqueue_gemm_group(a, &w, &c, &p->weight_offset, 1, p, x, stream);
 }
 
 } // namespace
@@ -831,6 +886,144 @@ int zdraw_hip_run_gemm(void* queue, void* pipeline, void* a, void* w, void* c, c
     return rc != ZDRAW_HIP_OK ? rc : rc2;
 }
 
+namespace {
+// Two or three products of the same f32 A (metal_api.m zdraw_metal_run_gemm_pair / _triple):
+// one grouped launch when the shapes and weight types agree, one launch each otherwise.
+int run_gemm_several(void* queue, void* pipeline, void* a, void* const* ws, void* const* cs,
+                     const ZdrawGemmParams* const* ps, int count) {
+    int rc = check_pipeline(pipeline, 0, 2);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    for (int i = 0; i < count; i++)
+        if (!ps[i]) {
+            set_err("null params");
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+    Batch* b = static_cast<Batch*>(zdraw_hip_batch_begin(queue));
+    if (!b) {
+        set_err("null queue");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    ZdrawHipGemmExt x;
+    memset(&x, 0, sizeof(x));
+    x.a_dtype = ZDRAW_HIP_F32;
+    x.c_dtype = ZDRAW_HIP_F32;
+    // a product this backend does not run refuses the call before anything is enqueued
+    for (int i = 0; i < count; i++) {
+        if (ps[i]->mode != ZDRAW_HIP_GEMM_HALF || (ps[i]->dtype != ZDRAW_HIP_W_F16 && ps[i]->dtype != ZDRAW_HIP_W_BF16) ||
+            (ps[i]->k % 8 != 0 && ps[i]->m != 0 && ps[i]->k != 0 && ps[i]->n != 0)) {
+            zdraw_hip_batch_end(b);
+            return unavailable("a product of the group is not a 16-bit-weight half-mode GEMM with k % 8 == 0");
+        }
+    }
+    bool same = true;
+    for (int i = 1; i < count; i++)
+        same = same && ps[i]->m == ps[0]->m && ps[i]->k == ps[0]->k && ps[i]->n == ps[0]->n &&
+               ps[i]->dtype == ps[0]->dtype && ps[i]->mode == ps[0]->mode;
+    if (same) {
+        uint64_t offs[3];
+        for (int i = 0; i < count; i++) offs[i] = ps[i]->weight_offset;
+        rc = enqueue_gemm_group(a, ws, cs, offs, count, ps[0], &x, b->queue->stream);
+    } else {
+        for (int i = 0; i < count && rc == ZDRAW_HIP_OK; i++) rc = enqueue_gemm(a, ws[i], cs[i], ps[i], &x, b->queue->stream);
+    }
+    const int rc2 = zdraw_hip_batch_end(b);
+    return rc != ZDRAW_HIP_OK ? rc : rc2;
+}
+} // namespace
+
+int zdraw_hip_run_gemm_pair(void* queue, void* pipeline, void* a, void* w0, void* c0, const ZdrawGemmParams* params0,
+                            void* w1, void* c1, const ZdrawGemmParams* params1) {
+    void* const ws[2] = {w0, w1};
+    void* const cs[2] = {c0, c1};
+    const ZdrawGemmParams* const ps[2] = {params0, params1};
+    return run_gemm_several(queue, pipeline, a, ws, cs, ps, 2);
+}
+
+int zdraw_hip_run_gemm_triple(void* queue, void* pipeline, void* a, void* w0, void* c0, const ZdrawGemmParams* params0,
+                              void* w1, void* c1, const ZdrawGemmParams* params1, void* w2, void* c2,
+                              const ZdrawGemmParams* params2) {
+    void* const ws[3] = {w0, w1, w2};
+    void* const cs[3] = {c0, c1, c2};
+    const ZdrawGemmParams* const ps[3] = {params0, params1, params2};
+    return run_gemm_several(queue, pipeline, a, ws, cs, ps, 3);
+}
+
+// ------------------------------------------------ Z-Image layer, attention segment
+int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bufs,
+                                 const ZdrawHipChainAttnWeights* w, const ZdrawHipChainAttnParams* p) {
+    Batch* b = static_cast<Batch*>(batch);
+    if (!b || !bufs || !w || !p) {
+        set_err("null argument");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    const ZdrawAttnParams& at = p->attn;
+    const uint64_t inner = (uint64_t)at.heads * at.head_dim;
+    // the segment's shapes must agree with each other before anything is enqueued
+    if (at.tokens == 0) return unavailable("tokens == 0");
+    if (p->q.m != at.tokens || p->k.m != at.tokens || p->v.m != at.tokens || p->proj.m != at.tokens)
+        return invalid("projection rows != attention tokens");
+    if (p->q.n != inner || p->k.n != (uint64_t)at.kv_heads * at.head_dim || p->v.n != p->k.n || p->proj.k != inner)
+        return invalid("projection widths != heads * head_dim");
+    if (p->k.k != p->q.k || p->v.k != p->q.k) return invalid("q/k/v projections read different widths");
+    if (p->qk.tokens != at.tokens || p->qk.heads != at.heads || p->qk.kv_heads != at.kv_heads || p->qk.head_dim != at.head_dim)
+        return invalid("QkNormParams shape != AttnParams shape");
+    if (p->act_dtype != ZDRAW_HIP_F32 && p->act_dtype != ZDRAW_HIP_BF16) return unavailable("activation dtype");
+    const ZdrawGemmParams* gs[4] = {&p->q, &p->k, &p->v, &p->proj};
+    for (const ZdrawGemmParams* g : gs) {
+        if (g->mode != ZDRAW_HIP_GEMM_HALF) return unavailable("only the half-precision GEMM mode exists");
+        if (g->dtype != ZDRAW_HIP_W_F16 && g->dtype != ZDRAW_HIP_W_BF16) return unavailable("weight dtype");
+        if (p->act_dtype == ZDRAW_HIP_BF16 && g->dtype != ZDRAW_HIP_W_BF16) return unavailable("bf16 activations need bf16 weights");
+        if (g->k % 8 != 0) return unavailable("k % 8 != 0");
+    }
+
+    ZdrawHipAttnExt x;
+    memset(&x, 0, sizeof(x));
+    const uint64_t row = inner;
+    x.q_stride[0] = x.k_stride[0] = x.v_stride[0] = x.out_stride[0] = (uint64_t)at.tokens * row;
+    x.q_stride[1] = x.k_stride[1] = x.v_stride[1] = x.out_stride[1] = row;
+    x.q_stride[2] = x.k_stride[2] = x.v_stride[2] = x.out_stride[2] = at.head_dim;
+    x.batch = 1;
+    x.in_dtype = x.out_dtype = p->act_dtype;
+    x.qk_mode = ZDRAW_HIP_QK_ZIMAGE;
+    x.k_site = ZDRAW_HIP_K_PREPASS;
+    x.eps = p->qk.eps;
+    x.score_bound = p->score_bound;
+    x.zimage_dims[0] = p->qk.dim0; x.zimage_dims[1] = p->qk.dim1; x.zimage_dims[2] = p->qk.dim2;
+    x.zimage_base[0] = p->qk.base0; x.zimage_base[1] = p->qk.base1; x.zimage_base[2] = p->qk.base2;
+    ZdrawHipQkOperands ops;
+    memset(&ops, 0, sizeof(ops));
+    ops.q_weight = w->q_norm;
+    ops.k_weight = w->k_norm;
+    ops.pos = w->pos;
+    ops.rope_pairs = w->rope;
+    const NormWeights nw{p->qk.q_dtype, p->qk.k_dtype, p->qk.q_offset, p->qk.k_offset};
+    FusedPlan plan;
+    int rc = plan_attention(b->queue->dev, bufs->q, bufs->k, bufs->v, bufs->mix, &at, &x, &ops, &plan, &nw);
+    if (rc != ZDRAW_HIP_OK) return rc;
+
+    ZdrawHipGemmExt gx;
+    memset(&gx, 0, sizeof(gx));
+    gx.a_dtype = gx.c_dtype = p->act_dtype;
+    hipStream_t st = b->queue->stream;
+    // a projection that is refused leaves nothing half-written that a later step
+    // reads: the caller re-runs the whole segment on its own path
+    // q, k and v read the same rows and have the same shape (kv_heads == heads was checked):
+    // one launch whose tiles cover all three, so the last partly filled round of workgroups
+    // is paid once instead of three times
+    if (p->k.dtype == p->q.dtype && p->v.dtype == p->q.dtype) {
+        void* const wsv[3] = {w->q, w->k, w->v};
+        void* const csv[3] = {bufs->q, bufs->k, bufs->v};
+        const uint64_t offs[3] = {p->q.weight_offset, p->k.weight_offset, p->v.weight_offset};
+        if ((rc = enqueue_gemm_group(bufs->norm, wsv, csv, offs, 3, &p->q, &gx, st)) != ZDRAW_HIP_OK) return rc;
+    } else {
+        if ((rc = enqueue_gemm(bufs->norm, w->q, bufs->q, &p->q, &gx, st)) != ZDRAW_HIP_OK) return rc;
+        if ((rc = enqueue_gemm(bufs->norm, w->k, bufs->k, &p->k, &gx, st)) != ZDRAW_HIP_OK) return rc;
+        if ((rc = enqueue_gemm(bufs->norm, w->v, bufs->v, &p->v, &gx, st)) != ZDRAW_HIP_OK) return rc;
+    }
+    if ((rc = enqueue(plan, st)) != ZDRAW_HIP_OK) return rc;
+    return enqueue_gemm(bufs->mix, w->proj, bufs->attn, &p->proj, &gx, st);
+}
+
 // ------------------------------------------------------------------ scratch
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes) {
     if (!device || slot < 0 || slot >= 5 || bytes == 0) return nullptr;
@@ -948,6 +1141,10 @@ size_t zdraw_hip_abi_sizeof(int which) {
     case 2: return sizeof(ZdrawHipQkOperands);
     case 3: return sizeof(ZdrawGemmParams);
     case 4: return sizeof(ZdrawHipGemmExt);
+    case 5: return sizeof(ZdrawQkNormParams);
+    case 6: return sizeof(ZdrawHipChainAttnBuffers);
+    case 7: return sizeof(ZdrawHipChainAttnWeights);
+    case 8: return sizeof(ZdrawHipChainAttnParams);
     default: return 0;
     }
 }

@@ -79,7 +79,7 @@ __device__ __forceinline__ f32x16 mfma(const u32x4& a, const u32x4& b, const f32
 
 // A wave's (32 TM) x (32 TN) block of C: lane holds column col0 + 32 j + l32, rows row0 + 32 i + 8 r + 4 h + jj.
 template <bool F16, typename TC, int TM, int TN>
-__device__ __forceinline__ void store_tile(const GemmArgs& g, const f32x16 (&acc)[TM][TN], int row0, int col0, int l32, int h) {
+__device__ __forceinline__ void store_tile(const GemmArgs& g, void* c, const f32x16 (&acc)[TM][TN], int row0, int col0, int l32, int h) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -92,7 +92,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs& g, const f32x16 (&acc
                     const int row = row0 + i * 32 + 8 * r + 4 * h + jj;
                     if (row < g.m && col < g.n) {
                         const float v = acc[i][j][4 * r + jj];
-                        TC* dst = reinterpret_cast<TC*>(g.c) + (int64_t)row * g.ldc + col;
+                        TC* dst = reinterpret_cast<TC*>(c) + (int64_t)row * g.ldc + col;
                         if constexpr (std::is_same<TC, float>::value) *dst = v;
                         else if constexpr (F16) *reinterpret_cast<_Float16*>(dst) = (_Float16)v;
                         else *reinterpret_cast<bf16_t*>(dst) = (bf16_t)v;
@@ -128,8 +128,14 @@ __global__ void __launch_bounds__(NT, 2) gemm_kernel(const GemmArgs g) {
     const int wm = wave >> 1, wn = wave & 1;
 
     const int logical = logical_tile();
-    const int tm = logical / g.tiles_n;
-    const int tn = logical - tm * g.tiles_n;
+    // the groups lie side by side along n: one row of tiles reads the same rows of A
+    const int tiles_row = g.tiles_n * g.groups;
+    const int tm = logical / tiles_row;
+    int tn = logical - tm * tiles_row;
+    const int grp = tn / g.tiles_n;
+    tn -= grp * g.tiles_n;
+    const void* const wp = grp == 0 ? g.w : g.w_more[grp - 1];
+    void* const cp = grp == 0 ? g.c : g.c_more[grp - 1];
     const int m0 = tm * BM, n0 = tn * BN;
 
     // ---- staging: thread t owns 16-byte chunk t%8 of rows t/8 + 64 j (j < 4) of the A slab and of the W slab
@@ -137,7 +143,7 @@ __global__ void __launch_bounds__(NT, 2) gemm_kernel(const GemmArgs g) {
     const unsigned a_span = ((unsigned)(g.m - 1) * (unsigned)g.lda + (unsigned)g.k) * ea;
     const unsigned w_span = ((unsigned)(g.n - 1) * (unsigned)g.ldw + (unsigned)g.k) * 2u;
     const rsrc_t a_rsrc = make_rsrc(g.a, a_span);
-    const rsrc_t w_rsrc = make_rsrc(g.w, w_span);
+    const rsrc_t w_rsrc = make_rsrc(wp, w_span);
     const int lr = tid >> 3;
     const int kc = tid & 7;
     unsigned a_off[4], w_off[4];
@@ -222,7 +228,7 @@ __global__ void __launch_bounds__(NT, 2) gemm_kernel(const GemmArgs g) {
         __syncthreads();
     }
 
-    store_tile<F16, TC, 2, 4>(g, acc, m0 + wm * 64, n0 + wn * 128, l32, h);
+    store_tile<F16, TC, 2, 4>(g, cp, acc, m0 + wm * 64, n0 + wn * 128, l32, h);
 }
 
 // The same tile with 16-bit activations and k a multiple of 64: both slabs go
@@ -254,14 +260,20 @@ __global__ void __launch_bounds__(WM * WN * 64, (WM * WN) / 4) gemm_dma_kernel(c
     const int h = lane >> 5;
     const int wm = wave / WN, wn = wave % WN;
     const int logical = logical_tile();
-    const int tm = logical / g.tiles_n;
-    const int tn = logical - tm * g.tiles_n;
+    // the groups lie side by side along n: one row of tiles reads the same rows of A
+    const int tiles_row = g.tiles_n * g.groups;
+    const int tm = logical / tiles_row;
+    int tn = logical - tm * tiles_row;
+    const int grp = tn / g.tiles_n;
+    tn -= grp * g.tiles_n;
+    const void* const wp = grp == 0 ? g.w : g.w_more[grp - 1];
+    void* const cp = grp == 0 ? g.c : g.c_more[grp - 1];
     const int m0 = tm * BM, n0 = tn * BN;
 
     const unsigned a_span = ((unsigned)(g.m - 1) * (unsigned)g.lda + (unsigned)g.k) * 2u;
     const unsigned w_span = ((unsigned)(g.n - 1) * (unsigned)g.ldw + (unsigned)g.k) * 2u;
     const rsrc_t a_rsrc = make_rsrc(g.a, a_span);
-    const rsrc_t w_rsrc = make_rsrc(g.w, w_span);
+    const rsrc_t w_rsrc = make_rsrc(wp, w_span);
     // wave w fills rows RW w + 8 j + lane / 8 (j < RW / 8) of the A slab and of the W slab
     unsigned a_off[RW / 8], w_off[RW / 8];
 #pragma unroll
@@ -328,7 +340,7 @@ __global__ void __launch_bounds__(WM * WN * 64, (WM * WN) / 4) gemm_dma_kernel(c
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): slab s+1 has landed
         __syncthreads();
     }
-    store_tile<F16, TC, TM, TN>(g, acc, m0 + wm * (32 * TM), n0 + wn * (32 * TN), l32, h);
+    store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * (32 * TM), n0 + wn * (32 * TN), l32, h);
 }
 
 // Measured on the Klein projections: 4 x 2 waves (two per SIMD, 64 x 128 each) 1090-1220
@@ -338,7 +350,7 @@ constexpr int DMA_WM = 4, DMA_WN = 2;
 template <typename TA, bool F16, typename TC>
 static hipError_t launch_one(const GemmArgs& g, hipStream_t stream) {
     const int64_t tiles_m = (g.m + BM - 1) / BM;
-    const int64_t nwg = tiles_m * g.tiles_n;
+    const int64_t nwg = tiles_m * g.tiles_n * g.groups;
     if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
     if constexpr (!std::is_same<TA, float>::value) {
         if (g.k % BK == 0) { // whole slabs of 16-bit activations: the direct-to-LDS build

@@ -15,8 +15,10 @@ struct GemmArgs {
     int32_t m, n, k;
     int32_t pad0;
     int64_t lda, ldw, ldc;
-    int32_t tiles_n; // column tiles (grid = tiles_m * tiles_n)
-    int32_t pad1;
+    int32_t tiles_n; // column tiles of one group (grid = tiles_m * tiles_n * groups)
+    int32_t groups;  // 1..3 products sharing A and every dimension: group i > 0 uses w_more[i-1], c_more[i-1]
+    const void* w_more[2];
+    void* c_more[2];
 };
 
 int gemm_tile_rows();

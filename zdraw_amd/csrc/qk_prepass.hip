@@ -42,11 +42,34 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
         const int head = h0 + 4 * g;
         raw[g] = ld_raw8<TIn>(src + (int64_t)(head < p.heads ? head : p.heads - 1) * p.x_hs, true);
     }
-    const QkRow qr = qk_row(p.qk, MODE, p.w, p.w_txt, seg, tok, true);
+    const QkRow qr = qk_row(p.qk, MODE, nullptr, nullptr, seg, tok, true);
     const Rope8 t = ld_rope8(p.qk, MODE, qr, d0);
     // the token's weights and rope row stay in registers across its heads
-    const f32x4 w0 = *reinterpret_cast<const f32x4*>(qr.w + d0);
-    const f32x4 w1 = *reinterpret_cast<const f32x4*>(qr.w + d0 + 4);
+    const void* wsel = (p.w_txt != nullptr && tok < p.qk.txt_rows) ? p.w_txt : p.w;
+    f32x4 w0, w1;
+    if (p.w_dtype == kF32) {
+        const float* wf = static_cast<const float*>(wsel) + d0;
+        w0 = *reinterpret_cast<const f32x4*>(wf);
+        w1 = *reinterpret_cast<const f32x4*>(wf + 4);
+    } else {
+        const u32x4 r = *reinterpret_cast<const u32x4*>(static_cast<const unsigned short*>(wsel) + d0);
+        float wv[8];
+        if (p.w_dtype == kBF16) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                wv[2 * i] = __builtin_bit_cast(float, r[i] << 16);
+                wv[2 * i + 1] = __builtin_bit_cast(float, r[i] & 0xffff0000u);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                wv[2 * i] = (float)__builtin_bit_cast(_Float16, (unsigned short)(r[i] & 0xffffu));
+                wv[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(r[i] >> 16));
+            }
+        }
+        w0 = f32x4{wv[0], wv[1], wv[2], wv[3]};
+        w1 = f32x4{wv[4], wv[5], wv[6], wv[7]};
+    }
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int head = h0 + 4 * g;

@@ -53,6 +53,31 @@ class GemmExt(C.Structure):
                 ("ldc", C.c_uint64), ("a_dtype", C.c_uint32), ("c_dtype", C.c_uint32)]
 
 
+class QkNormParams(C.Structure):
+    """ZdrawQkNormParams (metal_c.zig:258-274)"""
+    _fields_ = [("tokens", C.c_uint32), ("heads", C.c_uint32), ("kv_heads", C.c_uint32), ("head_dim", C.c_uint32),
+                ("q_dtype", C.c_uint32), ("k_dtype", C.c_uint32),
+                ("dim0", C.c_uint32), ("dim1", C.c_uint32), ("dim2", C.c_uint32), ("eps", C.c_float),
+                ("q_offset", C.c_uint64), ("k_offset", C.c_uint64),
+                ("base0", C.c_uint64), ("base1", C.c_uint64), ("base2", C.c_uint64)]
+
+
+class ChainAttnBuffers(C.Structure):
+    """ZdrawHipChainAttnBuffers"""
+    _fields_ = [(n, C.c_void_p) for n in ("norm", "q", "k", "v", "mix", "attn")]
+
+
+class ChainAttnWeights(C.Structure):
+    """ZdrawHipChainAttnWeights"""
+    _fields_ = [(n, C.c_void_p) for n in ("q", "k", "v", "q_norm", "k_norm", "pos", "rope", "proj")]
+
+
+class ChainAttnParams(C.Structure):
+    """ZdrawHipChainAttnParams"""
+    _fields_ = [("q", GemmParams), ("k", GemmParams), ("v", GemmParams), ("qk", QkNormParams),
+                ("attn", AttnParams), ("proj", GemmParams), ("act_dtype", C.c_uint32), ("score_bound", C.c_float)]
+
+
 W_F16, W_BF16, W_F32 = 1, 2, 3     # weight dtype codes of GemmParams.dtype
 GEMM_EXACT, GEMM_HALF = 1, 2       # GemmParams.mode
 
@@ -96,7 +121,11 @@ SYMBOLS = {
     "zdraw_hip_run_gemm_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _GP]),
     "zdraw_hip_run_gemm_off_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _GP, _u64, _u64]),
     "zdraw_hip_run_gemm_f16a_enc": (_int, [_vp, _vp, _vp, _vp, _GP, _u64, _u64]),
+    "zdraw_hip_run_gemm_pair": (_int, [_vp, _vp, _vp, _vp, _vp, _GP, _vp, _vp, _GP]),
+    "zdraw_hip_run_gemm_triple": (_int, [_vp, _vp, _vp, _vp, _vp, _GP, _vp, _vp, _GP, _vp, _vp, _GP]),
     "zdraw_hip_run_gemm_ext_enc": (_int, [_vp, _vp, _vp, _vp, _GP, _GX]),
+    "zdraw_hip_run_chain_attn_enc": (_int, [_vp, C.POINTER(ChainAttnBuffers), C.POINTER(ChainAttnWeights),
+                                            C.POINTER(ChainAttnParams)]),
     "zdraw_hip_mfma_probe": (_int, [_int, _int, C.POINTER(C.c_double)]),
     "zdraw_hip_clock_probe": (None, [_int]),
     "zdraw_hip_clock_probe_read": (C.c_size_t, [C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_size_t]),
