@@ -261,10 +261,96 @@ def chain_main(args):
     print(json.dumps(line), flush=True)
 
 
+def wide_main(args):
+    """`--path wide`: one wide head (heads 1, head_dim 512) at the VAE mid-block shape of a 1024 px
+    render, 16384 tokens, f32 token-major in and out as the reference passes them. The step is the
+    rounding pass + the attention kernel; FLOPs = 4 x 512 x tokens^2."""
+    import numpy as np
+
+    from zdraw_amd import hip, host
+
+    L = hip.lib()
+    ctx = host.Context.init()
+    tokens = args.wide_tokens
+    rng = np.random.default_rng(0)
+    q, k, v = (rng.standard_normal((tokens, 512), dtype=np.float32) for _ in range(3))
+    qb, kb, vb = ctx.buffer(q), ctx.buffer(k), ctx.buffer(v)
+    ob = ctx.buffer(nbytes=q.nbytes)
+    err = C.create_string_buffer(128)
+    pipe = L.zdraw_hip_compile(ctx.device, b"attention_wide_mfma", err, 128)
+    if not pipe:
+        raise RuntimeError(err.value)
+    p = hip.AttnParams(tokens, 1, 1, 512, 0, 0)
+
+    def burst(count):
+        b = L.zdraw_hip_batch_begin(ctx.queue)
+        for _ in range(count):
+            rc = L.zdraw_hip_run_attention_enc(b, pipe, qb.handle, kb.handle, vb.handle, ob.handle, C.byref(p),
+                                               hip.K_WIDE, 512)
+            if rc != 0:
+                raise RuntimeError(f"wide rc={rc}: {hip.last_error()}")
+        if L.zdraw_hip_batch_end(b) != 0:
+            raise RuntimeError("batch_end failed")
+
+    t0 = time.perf_counter()
+    spun = 0
+    while (time.perf_counter() - t0) * 1e3 < args.spinup_ms:
+        burst(20)
+        spun += 20
+    burst(max(args.warmup, 1))
+    L.zdraw_hip_queue_sync(ctx.queue)
+    t0 = time.perf_counter()
+    burst(args.steps)
+    wall = time.perf_counter() - t0
+    # the attention kernel alone: its own HIP events on the launch stream
+    L.zdraw_hip_trace_attention(1)
+    burst(args.steps)
+    launches = C.c_uint64(0)
+    ns = L.zdraw_hip_trace_attention_ns(C.byref(launches))
+    L.zdraw_hip_trace_attention(0)
+    kern_ms = ns / max(launches.value, 1) / 1e6
+    out = ob.read(np.float32, (tokens, 512))
+    if not np.isfinite(out).all():
+        raise RuntimeError("non-finite output")
+    flops = 4.0 * 512 * tokens * tokens
+    value = flops / (wall / args.steps) / 1e12
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+    line = {
+        "metric": "wide-head attention TFLOP/s (heads 1, head_dim 512)",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"vae mid-block attention: tokens {tokens}, heads 1, head_dim 512, f32 in and out",
+                   "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS, "untimed_spinup_launches": spun},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "attn_wide_kernel",
+                     "kernel_ms": kern_ms},
+    }
+    if not args.no_cpu:
+        from oracle import zoracle as zo
+        rows = list(range(0, tokens, max(tokens // 64, 1)))[:64]
+        t0 = time.perf_counter()
+        want = zo.attention_token_list(q.reshape(tokens, 1, 512), k.reshape(tokens, 1, 512), v.reshape(tokens, 1, 512),
+                                       zo.Config(tokens, 1, 1, 512), rows, threads=1)
+        dt = time.perf_counter() - t0
+        err_max = float(np.abs(out[rows] - want.reshape(len(rows), 512)).max())
+        if err_max > 2e-2:
+            raise RuntimeError(f"wide attention differs from the oracle on sampled rows: {err_max}")
+        line["cpu_baseline"] = {"value": 4.0 * 512 * len(rows) * tokens / dt / 1e12, "unit": "TFLOP/s", "cores": 1,
+                                "kind": "port", "sample": f"{len(rows)} of {tokens} query rows in {dt:.1f} s (max abs "
+                                f"difference from the GPU rows {err_max:.1e}); full call extrapolates to {dt / len(rows) * tokens:.0f} s"}
+    L.zdraw_hip_release_pipeline(pipe)
+    for b in (qb, kb, vb, ob):
+        b.release()
+    ctx.deinit()
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--path", choices=["attention", "gemm", "chain"], default="attention",
+    ap.add_argument("--path", choices=["attention", "gemm", "chain", "wide"], default="attention",
                     help="attention (the headline metric) or the projection GEMM beside it")
+    ap.add_argument("--wide-tokens", type=int, default=16384, help="--path wide: sequence length (multiple of 64)")
     ap.add_argument("--m", type=int, default=4608)
     ap.add_argument("--k", type=int, default=3072)
     ap.add_argument("--n", type=int, default=9216)
@@ -290,6 +376,8 @@ def main():
         return gemm_main(args)
     if args.path == "chain":
         return chain_main(args)
+    if args.path == "wide":
+        return wide_main(args)
 
     import numpy as np
 

@@ -96,6 +96,29 @@ struct PrepPair {
 int attention_block_rows(int shape);
 int attention_key_block();
 int attention_max_tokens();
+// One wide head (heads = 1, head_dim = 512), dense token-major rows.
+struct WideArgs {
+    const void* q; // bf16 [tokens][512], already multiplied by log2(e)/sqrt(512)
+    const void* k; // bf16 [tokens][512]
+    const void* v; // bf16 [tokens][512]
+    float* o;      // f32 [tokens][512]
+    int32_t tokens; // multiple of 64
+    int32_t pad0;
+};
+// f32 -> bf16 rounding of the three operands (Q with its scale) in one launch.
+struct WidePrepArgs {
+    const float* q; const float* k; const float* v;
+    void* qo; void* ko; void* vo;
+    int64_t chunks; // 8-element chunks per operand
+    float q_scale;
+    int32_t pad0;
+};
+int wide_head_dim();
+int wide_block_rows();
+hipError_t launch_wide_round(const WidePrepArgs& args, hipStream_t stream);
+hipError_t launch_wide_attention(const WideArgs& args, hipStream_t stream);
+hipError_t wide_setup();
+
 // Launch one attention forward. in_dtype is kF32 or kBF16; k_mode is the
 // QkMode applied to K rows inside the K-block load. Returns a hipError_t.
 hipError_t launch_attention(const AttnArgs& args, int in_dtype, int k_mode, int shape, hipStream_t stream);

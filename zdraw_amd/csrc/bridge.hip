@@ -443,6 +443,80 @@ int check_pipeline(void* pipeline, uint32_t kernel, int want_kind) {
         return ZDRAW_HIP_ERR_HANDLE;
     }
     if (want_kind == 0 && kernel != ZDRAW_HIP_K_BLOCK) return unavailable("only the block (MFMA) kernel exists");
+    if (want_kind == 3 && kernel != ZDRAW_HIP_K_WIDE) return unavailable("the wide pipeline runs the wide kernel only");
+    return ZDRAW_HIP_OK;
+}
+
+bool g_wide_setup_done = false;
+
+// One wide head (metal/mattn.zig:261-275 widePick, :280-283 sdpaShape): f32 token-major
+// q, k, v, out [tokens][512] at byte offsets; rounds the operands into scratch slots 0-2,
+// then runs the wide kernel.
+int enqueue_wide(Device* dev, void* q, void* k, void* v, void* out, const ZdrawAttnParams* p, uint64_t in_off,
+                 uint64_t out_off, hipStream_t stream) {
+    if (p->tokens == 0) return unavailable("tokens == 0");
+    if (p->heads != 1 || p->kv_heads != 1) return unavailable("the wide kernel runs one head");
+    if (p->head_dim != (uint32_t)wide_head_dim()) return unavailable("the wide kernel runs head_dim 512");
+    if (p->causal != 0) return unavailable("causal attention");
+    if (p->valid != 0 && p->valid != p->tokens) return unavailable("the wide kernel has no key limit");
+    if (p->tokens % (uint32_t)wide_block_rows() != 0) return unavailable("tokens % 64 != 0");
+    if (p->tokens > (1u << 20)) return unavailable("too many tokens");
+    const uint64_t n = (uint64_t)p->tokens * p->head_dim;
+    const Buffer* bs[4] = {static_cast<Buffer*>(q), static_cast<Buffer*>(k), static_cast<Buffer*>(v), static_cast<Buffer*>(out)};
+    for (int i = 0; i < 4; i++) {
+        const uint64_t off = i == 3 ? out_off : in_off;
+        if (!bs[i] || !bs[i]->ptr) return invalid("null buffer");
+        if (off % 16 != 0 || ((uintptr_t)bs[i]->ptr % 16) != 0) return invalid("operand not 16-byte aligned");
+        if (off > bs[i]->len || n * 4 > bs[i]->len - off) return invalid("buffer smaller than [tokens][512] f32");
+    }
+    Buffer* sc[3];
+    for (int i = 0; i < 3; i++) {
+        sc[i] = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, i, (size_t)n * 2));
+        if (!sc[i]) {
+            set_err("scratch allocation failed");
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+    }
+    if (!g_wide_setup_done) {
+        hipError_t e = wide_setup();
+        if (e != hipSuccess) {
+            set_err("wide_setup: %s", hipGetErrorString(e));
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        g_wide_setup_done = true;
+    }
+    WidePrepArgs pr;
+    memset(&pr, 0, sizeof(pr));
+    pr.q = reinterpret_cast<const float*>(static_cast<const char*>(bs[0]->ptr) + in_off);
+    pr.k = reinterpret_cast<const float*>(static_cast<const char*>(bs[1]->ptr) + in_off);
+    pr.v = reinterpret_cast<const float*>(static_cast<const char*>(bs[2]->ptr) + in_off);
+    pr.qo = sc[0]->ptr; pr.ko = sc[1]->ptr; pr.vo = sc[2]->ptr;
+    pr.chunks = (int64_t)(n / 8);
+    pr.q_scale = 1.4426950408889634f / sqrtf((float)p->head_dim);
+    hipError_t e = launch_wide_round(pr, stream);
+    if (e != hipSuccess) {
+        set_err("wide rounding launch: %s", hipGetErrorString(e));
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    g_dispatch++;
+    WideArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = sc[0]->ptr; a.k = sc[1]->ptr; a.v = sc[2]->ptr;
+    a.o = reinterpret_cast<float*>(static_cast<char*>(bs[3]->ptr) + out_off);
+    a.tokens = (int32_t)p->tokens;
+    TracePair tp{nullptr, nullptr};
+    if (g_trace && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
+        (void)hipEventRecord(tp.a, stream);
+    e = launch_wide_attention(a, stream);
+    if (e != hipSuccess) {
+        set_err("wide attention launch: %s", hipGetErrorString(e));
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    if (tp.a && tp.b) {
+        (void)hipEventRecord(tp.b, stream);
+        g_trace_open.push_back(tp);
+    }
+    g_dispatch++;
     return ZDRAW_HIP_OK;
 }
 
@@ -659,6 +733,7 @@ void* zdraw_hip_compile(void* device, const char* entry, char* error_buf, size_t
     if (strcmp(entry, "attention_block_mfma") == 0) return new Pipeline{0};
     if (strcmp(entry, "qk_norm_rope") == 0) return new Pipeline{1};
     if (strcmp(entry, "gemm_half") == 0) return new Pipeline{2};
+    if (strcmp(entry, "attention_wide_mfma") == 0) return new Pipeline{3};
     if (error_buf && error_len) snprintf(error_buf, error_len, "no gfx950 kernel named '%s'", entry);
     return nullptr;
 }
@@ -668,7 +743,7 @@ void zdraw_hip_release_pipeline(void* pipeline) { delete static_cast<Pipeline*>(
 size_t zdraw_hip_pipeline_threads(void* pipeline) {
     Pipeline* p = static_cast<Pipeline*>(pipeline);
     if (!p) return 0;
-    if (p->kind == 2) return 512;
+    if (p->kind == 2 || p->kind == 3) return 512;
     return p->kind == 0 ? (g_variant == 0 ? 512 : 256) : 256;
 }
 
@@ -681,17 +756,20 @@ int zdraw_hip_run_attention(void* queue, void* pipeline, void* q, void* k, void*
         set_err("null queue or params");
         return ZDRAW_HIP_ERR_HANDLE;
     }
-    int rc = check_pipeline(pipeline, kernel, 0);
+    const bool wide = pipeline && static_cast<Pipeline*>(pipeline)->kind == 3;
+    int rc = check_pipeline(pipeline, kernel, wide ? 3 : 0);
     if (rc != ZDRAW_HIP_OK) return rc;
     ZdrawHipAttnExt x;
-    standalone_ext(params, 0, 0, &x);
     FusedPlan plan;
-    rc = plan_attention(qu->dev, q, k, v, output, params, &x, nullptr, &plan);
-    if (rc != ZDRAW_HIP_OK) return rc;
+    if (!wide) {
+        standalone_ext(params, 0, 0, &x);
+        rc = plan_attention(qu->dev, q, k, v, output, params, &x, nullptr, &plan);
+        if (rc != ZDRAW_HIP_OK) return rc;
+    }
     hipEvent_t start, stop;
     if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return ZDRAW_HIP_ERR_HANDLE;
     (void)hipEventRecord(start, qu->stream);
-    rc = enqueue(plan, qu->stream);
+    rc = wide ? enqueue_wide(qu->dev, q, k, v, output, params, 0, 0, qu->stream) : enqueue(plan, qu->stream);
     if (rc == ZDRAW_HIP_OK) rc = finish_blocking(qu, start, stop);
     (void)hipEventDestroy(start);
     (void)hipEventDestroy(stop);
@@ -719,8 +797,10 @@ int zdraw_hip_run_attention_enc_off(void* batch, void* pipeline, void* q, void* 
         set_err("null batch or params");
         return ZDRAW_HIP_ERR_HANDLE;
     }
-    int rc = check_pipeline(pipeline, kernel, 0);
+    const bool wide = pipeline && static_cast<Pipeline*>(pipeline)->kind == 3;
+    int rc = check_pipeline(pipeline, kernel, wide ? 3 : 0);
     if (rc != ZDRAW_HIP_OK) return rc;
+    if (wide) return enqueue_wide(b->queue->dev, q, k, v, o, params, in_off, out_off, b->queue->stream);
     ZdrawHipAttnExt x;
     standalone_ext(params, in_off, out_off, &x);
     FusedPlan plan;

@@ -59,6 +59,8 @@ Error Context::initKernel(Kernel kernel, Context* out) {
         return Error::CompileFailed;
     }
     c.qk_pipeline = zdraw_hip_compile(c.device, "qk_norm_rope", err, sizeof(err)); // optional, like mattn.zig:86
+    c.wide_pipeline = zdraw_hip_compile(c.device, "attention_wide_mfma", err, sizeof(err)); // optional, mattn.zig:83-85
+    c.wide_threads = c.wide_pipeline ? zdraw_hip_pipeline_threads(c.wide_pipeline) : 0;
     c.kernel = kernel;
     c.threads = zdraw_hip_pipeline_threads(c.block_pipeline);
     c.qk_threads = c.qk_pipeline ? zdraw_hip_pipeline_threads(c.qk_pipeline) : 0;
@@ -72,6 +74,7 @@ void Context::deinit() {
         pool[i] = nullptr;
         pool_bytes[i] = 0;
     }
+    if (wide_pipeline) zdraw_hip_release_pipeline(wide_pipeline);
     if (qk_pipeline) zdraw_hip_release_pipeline(qk_pipeline);
     if (block_pipeline) zdraw_hip_release_pipeline(block_pipeline);
     if (queue) zdraw_hip_release_queue(queue);
@@ -86,6 +89,16 @@ bool Context::pick(size_t tokens, size_t head_dim, Pick* out) const {
     // there is none for other widths.
     if (head_dim != flash_head_dim || !block_pipeline) return false;
     *out = Pick{Kernel::block, block_pipeline, threads};
+    return true;
+}
+
+// mattn.zig:261-275 (widePick): one head of width 512 in whole 64-row blocks. The
+// reference keeps its wide kernel behind an opt-in switch because it lost to the
+// system's graph route there; here it is the only route for the shape, at any length.
+bool Context::widePick(const attention::Config& cfg, Pick* out) const {
+    if (!wide_pipeline || cfg.heads != 1 || cfg.kv_heads != 1 || cfg.causal) return false;
+    if (cfg.head_dim != wide_head_dim || cfg.tokens == 0 || cfg.tokens % 64 != 0 || cfg.valid != 0) return false;
+    *out = Pick{Kernel::wide, wide_pipeline, wide_threads};
     return true;
 }
 
@@ -128,10 +141,13 @@ bool paramsFor(const attention::Config& cfg, ZdrawAttnParams* p) {
 
 Error Context::run(float* out, size_t out_len, const float* q, size_t q_len, const float* k, size_t k_len,
                    const float* v, size_t v_len, const attention::Config& cfg) {
-    Error e = check(out_len, q_len, k_len, v_len, cfg);
-    if (e != Error::Ok) return e;
     Pick picked;
-    if (!pick(cfg.tokens, cfg.head_dim, &picked)) return Error::UnsupportedShape;
+    const bool wide = widePick(cfg, &picked);
+    // mattn.zig:320-331 (checkWide) adds nothing to widePick but the length check; every other shape
+    // takes check()
+    Error e = wide ? checkLens(out_len, q_len, k_len, v_len, cfg) : check(out_len, q_len, k_len, v_len, cfg);
+    if (e != Error::Ok) return e;
+    if (!wide && !pick(cfg.tokens, cfg.head_dim, &picked)) return Error::UnsupportedShape;
     // Causal and grouped-query shapes belong to the text encoder; the backend
     // refuses them before anything is uploaded.
     if (cfg.causal || cfg.kv_heads != cfg.heads) return Error::UnsupportedShape;
@@ -159,10 +175,13 @@ Error Context::run(float* out, size_t out_len, const float* q, size_t q_len, con
 
 Error Context::runPooled(float* out, size_t out_len, const float* q, size_t q_len, const float* k, size_t k_len,
                          const float* v, size_t v_len, const attention::Config& cfg) {
-    Error e = check(out_len, q_len, k_len, v_len, cfg);
-    if (e != Error::Ok) return e;
     Pick picked;
-    if (!pick(cfg.tokens, cfg.head_dim, &picked)) return Error::UnsupportedShape;
+    const bool wide = widePick(cfg, &picked);
+    // mattn.zig:320-331 (checkWide) adds nothing to widePick but the length check; every other shape
+    // takes check()
+    Error e = wide ? checkLens(out_len, q_len, k_len, v_len, cfg) : check(out_len, q_len, k_len, v_len, cfg);
+    if (e != Error::Ok) return e;
+    if (!wide && !pick(cfg.tokens, cfg.head_dim, &picked)) return Error::UnsupportedShape;
     if (cfg.causal || cfg.kv_heads != cfg.heads) return Error::UnsupportedShape;
     ZdrawAttnParams params;
     if (!paramsFor(cfg, &params)) return Error::InvalidShape;
@@ -190,7 +209,7 @@ Error Context::runOnHandles(void* q_h, void* k_h, void* v_h, void* out_h, const 
     ZdrawAttnParams params;
     if (!paramsFor(cfg, &params)) return Error::InvalidShape;
     Pick picked;
-    if (!pick(cfg.tokens, cfg.head_dim, &picked)) return Error::UnsupportedShape;
+    if (!widePick(cfg, &picked) && !pick(cfg.tokens, cfg.head_dim, &picked)) return Error::UnsupportedShape;
     const int code = zdraw_hip_run_attention(queue, picked.pipeline, q_h, k_h, v_h, out_h, &params,
                                              (uint32_t)picked.kernel, picked.threads);
     return fromCode(code);

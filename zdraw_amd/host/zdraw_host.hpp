@@ -53,6 +53,7 @@ namespace hattn {
 
 constexpr size_t max_tokens = 32768;    // key-block list capacity of the kernel (mattn.zig:15 is 6144 for `rows`)
 constexpr size_t flash_head_dim = 128;  // mattn.zig:16
+constexpr size_t wide_head_dim = 512;   // mattn.zig:17
 
 // mattn.zig:19. Only `block` (the bf16-MFMA flash kernel) exists on gfx950.
 enum class Kernel : uint32_t { rows = 0, flash = 1, block = 2, wide = 3 };
@@ -79,6 +80,8 @@ struct Context {
     void* queue = nullptr;
     void* block_pipeline = nullptr;
     void* qk_pipeline = nullptr;
+    void* wide_pipeline = nullptr; // one head of width 512 (the VAE mid-block), mattn.zig:53
+    size_t wide_threads = 0;
     Kernel kernel = Kernel::block;
     size_t threads = 0;
     size_t qk_threads = 0;
@@ -90,6 +93,7 @@ struct Context {
     static Error initKernel(Kernel kernel, Context* out);  // mattn.zig:69-118
     void deinit();                                         // mattn.zig:120-130
     bool pick(size_t tokens, size_t head_dim, Pick* out) const; // mattn.zig:134-150; false = no kernel for the shape
+    bool widePick(const attention::Config& cfg, Pick* out) const; // mattn.zig:261-275
 
     // mattn.zig:152-173: host f32 token-major slices in, out.
     Error run(float* out, size_t out_len, const float* q, size_t q_len, const float* k, size_t k_len,
