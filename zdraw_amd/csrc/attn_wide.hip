@@ -37,11 +37,10 @@ constexpr int NW = 8;
 constexpr int NT = NW * 64;
 constexpr int BQ = 64;            // query rows per workgroup
 constexpr int TILE_BYTES = KB * SL * 2;            // one slice of a K (or V) block: 8 KB
-constexpr int SLICE_BYTES = 2 * TILE_BYTES;        // K then V
-constexpr int STAGE_BYTES = NSL * SLICE_BYTES;     // 64 KB
-constexpr int NSTAGE = 2;
+constexpr int RING_BYTES = NSL * TILE_BYTES;       // one K (or V) block, all slices: 32 KB
+constexpr int V_RING = 2 * RING_BYTES;             // two K slots, then two V slots
 constexpr int X_BYTES = 2 * NSL * 64 * 16 * 4;     // partial scores: [group][slice][4 x (lane x 16 B)]: 32 KB
-constexpr size_t kLdsBytes = (size_t)NSTAGE * STAGE_BYTES + X_BYTES;
+constexpr size_t kLdsBytes = (size_t)4 * RING_BYTES + X_BYTES;
 constexpr float kTau = 8.0f;      // log2 headroom of the lazy softmax maximum
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -78,7 +77,7 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
     const int nblk = a.tokens / KB;
 
     const unsigned lds0 = lds_address(smem);
-    const unsigned xbase = lds0 + NSTAGE * STAGE_BYTES;
+    const unsigned xbase = lds0 + 4 * RING_BYTES;
 
     // ---- Q fragments (B operand): query q0 + l32, dims 128 sl + 16 kk + 8 h .. +7
     bf16x8 qf[8];
@@ -88,10 +87,11 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
         for (int kk = 0; kk < 8; kk++) qf[kk] = *reinterpret_cast<const bf16x8*>(qp + 16 * kk);
     }
 
-    // ---- block fetch: wave w fills rows 16 (w >> 2) .. +15 of slice w & 3, K and V, four
-    // rows per instruction. The lane that fills chunk position p of row r fetches the chunk
-    // the swizzle places there: K chunk c of row r sits at c ^ (r & 15), V chunk c at
-    // c ^ ((r & 3) << 2).
+    // ---- block fetch: wave w fills rows 16 (w >> 2) .. +15 of slice w & 3 of a K block or of a
+    // V block, four rows per instruction. The lane that fills chunk position p of row r
+    // fetches the chunk the swizzle places there: K chunk c of row r sits at c ^ (r & 15),
+    // V chunk c at c ^ ((r & 3) << 2). Positions past the last block re-fetch the last block
+    // into a slot nobody reads any more.
     const unsigned span = (unsigned)a.tokens * (unsigned)(WD * 2);
     const u32x4 k_rsrc = make_rsrc_words(a.k, span);
     const u32x4 v_rsrc = make_rsrc_words(a.v, span);
@@ -104,27 +104,30 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
         fk_off[j] = (unsigned)row * (WD * 2) + (unsigned)sl * (SL * 2) + kc * 16u;
         fv_off[j] = (unsigned)row * (WD * 2) + (unsigned)sl * (SL * 2) + vc * 16u;
     }
-    const unsigned fetch_lds = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)sl * SLICE_BYTES + (unsigned)(16 * grp) * (SL * 2));
-    auto fetch = [&](int blk, int stage) __attribute__((always_inline)) {
-        const unsigned uo = (unsigned)blk * (unsigned)(KB * WD * 2);
-        const unsigned base = fetch_lds + (unsigned)stage * STAGE_BYTES;
+    const unsigned fetch_lds = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)sl * TILE_BYTES + (unsigned)(16 * grp) * (SL * 2));
+    auto fetch_k = [&](int blk, int slot) __attribute__((always_inline)) {
+        const unsigned uo = (unsigned)(blk < nblk ? blk : nblk - 1) * (unsigned)(KB * WD * 2);
+        const unsigned base = fetch_lds + (unsigned)slot * RING_BYTES;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            load_to_lds_16(k_rsrc, base + (unsigned)(4 * j) * (SL * 2), fk_off[j], uo);
-            load_to_lds_16(v_rsrc, base + TILE_BYTES + (unsigned)(4 * j) * (SL * 2), fv_off[j], uo);
-        }
+        for (int j = 0; j < 4; j++) load_to_lds_16(k_rsrc, base + (unsigned)(4 * j) * (SL * 2), fk_off[j], uo);
+    };
+    auto fetch_v = [&](int blk, int slot) __attribute__((always_inline)) {
+        const unsigned uo = (unsigned)(blk < nblk ? blk : nblk - 1) * (unsigned)(KB * WD * 2);
+        const unsigned base = fetch_lds + V_RING + (unsigned)slot * RING_BYTES;
+#pragma unroll
+        for (int j = 0; j < 4; j++) load_to_lds_16(v_rsrc, base + (unsigned)(4 * j) * (SL * 2), fv_off[j], uo);
     };
 
-    // ---- fragment addresses in stage 0 (a stage adds a constant)
+    // ---- fragment addresses in slot 0 of each ring (a slot adds a constant)
     const int tr_row = (lane & 15) >> 2;
     const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     unsigned kfo[8], vfo[4];
 #pragma unroll
     for (int kk = 0; kk < 8; kk++)
-        kfo[kk] = lds0 + (unsigned)sl * SLICE_BYTES + (unsigned)((l32 * SL + (((2 * kk + h) ^ (l32 & 15)) * 8)) * 2);
+        kfo[kk] = lds0 + (unsigned)sl * TILE_BYTES + (unsigned)((l32 * SL + (((2 * kk + h) ^ (l32 & 15)) * 8)) * 2);
 #pragma unroll
     for (int blk = 0; blk < 4; blk++)
-        vfo[blk] = lds0 + (unsigned)sl * SLICE_BYTES + TILE_BYTES +
+        vfo[blk] = lds0 + V_RING + (unsigned)sl * TILE_BYTES +
                    (unsigned)(((4 * h + tr_row) * SL + ((blk ^ tr_row) * 32) + tr_col) * 2);
     typedef const __attribute__((address_space(3))) bf16x8* lds_bf16x8_t;
     typedef __attribute__((address_space(3))) s16x4* lds_s16x4_t;
@@ -133,37 +136,13 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
     // partial-score exchange: [group][slice][i < 4][lane] x 16 B
     const unsigned x_mine = xbase + (unsigned)(((grp * NSL + sl) * 4) * 64 + lane) * 16u;
     const unsigned x_group = xbase + (unsigned)((grp * NSL * 4) * 64 + lane) * 16u;
-
-    f32x16 oacc[4]; // O^T slice: lane = query l32, dims 128 sl + 32 blk + 8 i + 4 h + j
-#pragma unroll
-    for (int blk = 0; blk < 4; blk++)
-#pragma unroll
-        for (int j = 0; j < 16; j++) oacc[blk][j] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-
-    fetch(0, 0);
-    if (nblk > 1) fetch(1, 1);
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-    __syncthreads();
-
-    for (int b = 0; b < nblk; b++) {
-        const unsigned so = (unsigned)(b & 1) * STAGE_BYTES;
-        // partial S^T = K_s(b) . Q_s^T: lane = query l32, element 4 i + j = key 8 i + 4 h + j
-        f32x16 sp;
-#pragma unroll
-        for (int j = 0; j < 16; j++) sp[j] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < 8; kk++) {
-            const bf16x8 kf = *(lds_bf16x8_t)(kfo[kk] + so);
-            sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], sp, 0, 0, 0);
-        }
+    auto x_write = [&](const f32x16& sp) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; i++)
             *(lds_f32x4_t)(x_mine + (unsigned)(i * 64 * 16)) = f32x4{sp[4 * i], sp[4 * i + 1], sp[4 * i + 2], sp[4 * i + 3]};
-        __syncthreads();
-
-        // full scores: ((p0 + p1) + p2) + p3, the same in each of the group's four waves
-        f32x16 sv;
+    };
+    // full scores: ((p0 + p1) + p2) + p3, the same in each of the group's four waves
+    auto x_sum = [&](f32x16& sv) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             f32x4 t = *(lds_f32x4_t)(x_group + (unsigned)((0 * 4 + i) * 64 * 16));
@@ -175,57 +154,127 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
 #pragma unroll
             for (int j = 0; j < 4; j++) sv[4 * i + j] = t[j];
         }
+    };
 
-        // online softmax in the exp2 domain (the scale rides on Q) with a lazy maximum: the
-        // reference point moves only when this block's maximum exceeds it by more than kTau
-        float mloc = sv[0];
+    f32x16 oacc[4]; // O^T slice: lane = query l32, dims 128 sl + 32 blk + 8 i + 4 h + j
 #pragma unroll
-        for (int j = 1; j < 16; j++) mloc = fmaxf(mloc, sv[j]);
-        const float mlc = pair_max(mloc);
-        const bool up = mlc > m_run + kTau;
-        const float m_new = up ? mlc : m_run;
-        const float mc = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - mc);
-        m_run = m_new;
-        float psum = 0.f;
+    for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) oacc[blk][j] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // ---- prologue: K(0), K(1), V(0) in; scores of block 0 exchanged; K(2), V(1) requested.
+    // K runs one block ahead of V: step b multiplies by K(b+1) and by V(b).
+    fetch_k(0, 0);
+    fetch_v(0, 0);
+    fetch_k(1, 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    __syncthreads();
+    f32x16 sv; // scores of the block the next step exponentiates: lane = query l32, element 4 i + j = key 8 i + 4 h + j
+    {
+        f32x16 sp;
+#pragma unroll
+        for (int j = 0; j < 16; j++) sp[j] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++)
+            sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(lds_bf16x8_t)(kfo[kk]), qf[kk], sp, 0, 0, 0);
+        x_write(sp);
+        __syncthreads();
+        x_sum(sv);
+        __syncthreads();
+    }
+    fetch_k(2, 0);
+    fetch_v(1, 1);
+
+    // One step: the MFMAs of S(b+1) = K(b+1) Q^T (this wave's slice) run with the softmax of
+    // block b in their shadow, then O += V(b)^T P(b)^T; the partial scores of block b+1 are
+    // published between the two, and collected after the barrier that also says "block
+    // b+2's K and block b+1's V have landed, K(b+1) and V(b) have no reader left".
+    for (int b = 0; b < nblk; b++) {
+        const unsigned kso = (unsigned)((b + 1) & 1) * RING_BYTES;
+        const unsigned vso = (unsigned)(b & 1) * RING_BYTES;
+        bf16x8 kf[8];
+        s16x4 vlo[8], vhi[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) kf[kk] = *(lds_bf16x8_t)(kfo[kk] + kso);
+        auto v_read = [&](int idx) __attribute__((always_inline)) {
+            const int kb = idx >> 2, blk = idx & 3;
+            const unsigned va = vfo[blk] + vso + (unsigned)(16 * kb) * (SL * 2);
+            vlo[idx] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)va);
+            vhi[idx] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(va + 8u * (SL * 2)));
+        };
+        f32x16 sp;
+#pragma unroll
+        for (int j = 0; j < 16; j++) sp[j] = 0.f;
+        float mloc = 0.f, mc = 0.f, alpha = 1.f, psum = 0.f;
+        bool up = false;
         unsigned pc[8];
-#pragma unroll
-        for (int pr = 0; pr < 8; pr++) {
+        auto exp_pair = [&](int pr) __attribute__((always_inline)) {
             f32x2 pp;
             pp[0] = __builtin_amdgcn_exp2f(sv[2 * pr] - mc);
             pp[1] = __builtin_amdgcn_exp2f(sv[2 * pr + 1] - mc);
             psum += pp[0] + pp[1];
             pc[pr] = __builtin_bit_cast(unsigned, __builtin_convertvector(pp, bf16x2));
-        }
-        l_run = l_run * alpha + psum;
-        if (__any(up)) {
+        };
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int blk = 0; blk < 4; blk++)
+        for (int g = 0; g < 8; g++) {
+            __builtin_amdgcn_s_setprio(1);
+            sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[g], qf[g], sp, 0, 0, 0);
+            __builtin_amdgcn_s_setprio(0);
+            // softmax of block b in the exp2 domain (the scale rides on Q) with a lazy maximum:
+            // the reference point moves only when this block's maximum exceeds it by more than kTau
+            if (g == 0) {
+                mloc = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+                v_read(0);
+                v_read(1);
+            } else if (g == 1) {
+                mloc = fmaxf(mloc, fmaxf(fmaxf(fmaxf(sv[8], sv[9]), fmaxf(sv[10], sv[11])), fmaxf(fmaxf(sv[12], sv[13]), fmaxf(sv[14], sv[15]))));
+                const float mlc = pair_max(mloc);
+                up = mlc > m_run + kTau;
+                const float m_new = up ? mlc : m_run;
+                mc = (m_new == -INFINITY) ? 0.f : m_new;
+                alpha = __builtin_amdgcn_exp2f(m_run - mc);
+                m_run = m_new;
+                v_read(2);
+                v_read(3);
+            } else if (g < 6) {
+                exp_pair(2 * (g - 2));
+                exp_pair(2 * (g - 2) + 1);
+                if (g < 4) {
+                    v_read(2 * g);
+                    v_read(2 * g + 1);
+                }
+            } else if (g == 6) {
+                l_run = l_run * alpha + psum;
+                if (__any(up)) {
 #pragma unroll
-                for (int j = 0; j < 16; j++) oacc[blk][j] *= alpha;
+                    for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                        for (int j = 0; j < 16; j++) oacc[blk][j] *= alpha;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
         const bf16x8 p0 = __builtin_bit_cast(bf16x8, u32x4{pc[0], pc[1], pc[2], pc[3]});
         const bf16x8 p1 = __builtin_bit_cast(bf16x8, u32x4{pc[4], pc[5], pc[6], pc[7]});
-
         // O^T slice += V_s(b)^T . P^T; the transposing read delivers keys in P's order
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-            for (int blk = 0; blk < 4; blk++) {
-                const unsigned va = vfo[blk] + so + (unsigned)(16 * kb) * (SL * 2);
-                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)va);
-                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(va + 8u * (SL * 2)));
-                const bf16x8 vf = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-                oacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, kb == 0 ? p0 : p1, oacc[blk], 0, 0, 0);
-            }
+        for (int idx = 0; idx < 8; idx++) {
+            const bf16x8 vf = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(vlo[idx], vhi[idx], 0, 1, 2, 3, 4, 5, 6, 7));
+            __builtin_amdgcn_s_setprio(1);
+            oacc[idx & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, idx < 4 ? p0 : p1, oacc[idx & 3], 0, 0, 0);
+            __builtin_amdgcn_s_setprio(0);
+            if (idx == 1) x_write(sp); // the S MFMAs have drained by now
+            __builtin_amdgcn_sched_barrier(0);
         }
-
-        // block b + 1 was requested a whole step ago; once every wave has seen its own part
-        // land and passed the barrier, the other stage is complete, and this stage and the
-        // exchange area have no reader left
+        // every wave has seen its own part of K(b+2) and V(b+1) land (requested a step ago)
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
-        if (b + 2 < nblk) fetch(b + 2, b & 1);
+        fetch_k(b + 3, (b + 1) & 1);
+        fetch_v(b + 2, b & 1);
+        x_sum(sv);
+        __syncthreads(); // the exchange area is rewritten in the next step
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
 
