@@ -644,6 +644,7 @@ void* zdraw_hip_create_device(void) {
     if (hipSetDevice(0) != hipSuccess) return nullptr;
     // ZDRAW_ATTN_VARIANT picks the kernel build for a whole process (measurement aid)
     if (const char* v = getenv("ZDRAW_ATTN_VARIANT")) zdraw_hip_set_attention_variant(atoi(v));
+    if (const char* v = getenv("ZDRAW_GEMM_BUILD")) gemm_set_build(atoi(v));
     Device* d = new Device{0};
     return d;
 }

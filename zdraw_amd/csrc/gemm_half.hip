@@ -77,25 +77,38 @@ __device__ __forceinline__ f32x16 mfma(const u32x4& a, const u32x4& b, const f32
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// A wave's (32 TM) x (32 TN) block of C: lane holds column col0 + 32 j + l32, rows row0 + 32 i + 8 r + 4 h + jj.
+// A wave's (32 TM) x (32 TN) block of C. The MFMAs take the W fragment as their first
+// operand, so a lane holds row row0 + 32 i + l32 of C and, in register 4 r + jj of tile
+// (i, j), column col0 + 32 j + 8 r + 4 h + jj: four consecutive columns per r, stored as
+// one 8- or 16-byte vector where the row pitch and the base allow it.
 template <bool F16, typename TC, int TM, int TN>
 __device__ __forceinline__ void store_tile(const GemmArgs& g, void* c, const f32x16 (&acc)[TM][TN], int row0, int col0, int l32, int h) {
+    // uniform over the launch: every group of four columns starts aligned for a vector store
+    const bool vec = (g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) % (4 * sizeof(TC))) == 0);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
+        const int row = row0 + i * 32 + l32;
+        if (row >= g.m) continue;
+        TC* const crow = reinterpret_cast<TC*>(c) + (int64_t)row * g.ldc;
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            const int col = col0 + j * 32 + l32;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
+                const int col = col0 + j * 32 + 8 * r + 4 * h;
+                const f32x4 v = f32x4{acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2], acc[i][j][4 * r + 3]};
+                if (vec && col + 3 < g.n) {
+                    if constexpr (std::is_same<TC, float>::value) *reinterpret_cast<f32x4*>(crow + col) = v;
+                    else if constexpr (F16) *reinterpret_cast<f16x4*>(crow + col) = __builtin_convertvector(v, f16x4);
+                    else *reinterpret_cast<bf16x4*>(crow + col) = __builtin_convertvector(v, bf16x4);
+                } else {
 #pragma unroll
-                for (int jj = 0; jj < 4; jj++) {
-                    const int row = row0 + i * 32 + 8 * r + 4 * h + jj;
-                    if (row < g.m && col < g.n) {
-                        const float v = acc[i][j][4 * r + jj];
-                        TC* dst = reinterpret_cast<TC*>(c) + (int64_t)row * g.ldc + col;
-                        if constexpr (std::is_same<TC, float>::value) *dst = v;
-                        else if constexpr (F16) *reinterpret_cast<_Float16*>(dst) = (_Float16)v;
-                        else *reinterpret_cast<bf16_t*>(dst) = (bf16_t)v;
+                    for (int jj = 0; jj < 4; jj++) {
+                        if (col + jj < g.n) {
+                            TC* dst = crow + col + jj;
+                            if constexpr (std::is_same<TC, float>::value) *dst = v[jj];
+                            else if constexpr (F16) *reinterpret_cast<_Float16*>(dst) = (_Float16)v[jj];
+                            else *reinterpret_cast<bf16_t*>(dst) = (bf16_t)v[jj];
+                        }
                     }
                 }
             }
@@ -213,7 +226,7 @@ __global__ void __launch_bounds__(NT, 2) gemm_kernel(const GemmArgs g) {
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = mfma<F16>(af[i], wf[j], acc[i][j]);
+                for (int j = 0; j < 4; j++) acc[i][j] = mfma<F16>(wf[j], af[i], acc[i][j]);
             if (kk == 0) {
                 // slab s+1 (in registers since the previous iteration) goes to the other stage,
                 // whose readers finished before the last barrier; then slab s+2 starts loading.
@@ -242,14 +255,15 @@ __global__ void __launch_bounds__(NT, 2) gemm_kernel(const GemmArgs g) {
 constexpr int DMA_STAGE_BYTES = (BM + BN) * BK * 2; // 64 KB
 constexpr size_t kDmaLdsBytes = 2 * (size_t)DMA_STAGE_BYTES;
 
-// WM x WN waves; a wave owns (256 / WM) x (256 / WN) of C. 4 x 2 waves run two per SIMD
-// with 64 x 128 each; 2 x 2 waves run one per SIMD with 128 x 128 each (256 accumulator
-// registers), which reads a third fewer LDS bytes per MFMA.
-template <bool F16, typename TC, int WM, int WN>
-__global__ void __launch_bounds__(WM * WN * 64, (WM * WN) / 4) gemm_dma_kernel(const GemmArgs g) {
+// TB x TB tile of C, WM x WN waves, a wave owns (TB / WM) x (TB / WN). Built as 256 with
+// 4 x 2 waves (two per SIMD, 64 x 128 each) and as 128 with 2 x 2 waves (64 x 64 each, 64 KB
+// of LDS, two workgroups per CU) for problems with too few 256-tiles to fill the chip.
+template <bool F16, typename TC, int WM, int WN, int TB>
+__global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArgs g) {
+    constexpr int STAGE_BYTES = 2 * TB * BK * 2; // A rows then W rows
     constexpr int NW = WM * WN;
-    constexpr int TM = BM / WM / 32, TN = BN / WN / 32; // 32 x 32 MFMA tiles per wave
-    constexpr int RW = BM / NW;                           // slab rows a wave fetches, of A and of W
+    constexpr int TM = TB / WM / 32, TN = TB / WN / 32; // 32 x 32 MFMA tiles per wave
+    constexpr int RW = TB / NW;                           // slab rows a wave fetches, of A and of W
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -268,7 +282,7 @@ __global__ void __launch_bounds__(WM * WN * 64, (WM * WN) / 4) gemm_dma_kernel(c
     tn -= grp * g.tiles_n;
     const void* const wp = grp == 0 ? g.w : g.w_more[grp - 1];
     void* const cp = grp == 0 ? g.c : g.c_more[grp - 1];
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = tm * TB, n0 = tn * TB;
 
     const unsigned a_span = ((unsigned)(g.m - 1) * (unsigned)g.lda + (unsigned)g.k) * 2u;
     const unsigned w_span = ((unsigned)(g.n - 1) * (unsigned)g.ldw + (unsigned)g.k) * 2u;
@@ -287,12 +301,12 @@ __global__ void __launch_bounds__(WM * WN * 64, (WM * WN) / 4) gemm_dma_kernel(c
     }
     const int nslab = g.k / BK;
     auto fetch_slab = [&](int s) __attribute__((always_inline)) {
-        unsigned char* st = smem + (s & 1) * DMA_STAGE_BYTES + wave * (RW * BK * 2);
+        unsigned char* st = smem + (s & 1) * STAGE_BYTES + wave * (RW * BK * 2);
 #pragma unroll
         for (int j = 0; j < RW / 8; j++) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (lds_ptr_t)(st + j * (8 * BK * 2)), 16, (int)a_off[j],
                                                      (int)((unsigned)s * (BK * 2u)), 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr_t)(st + BM * BK * 2 + j * (8 * BK * 2)), 16,
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr_t)(st + TB * BK * 2 + j * (8 * BK * 2)), 16,
                                                      (int)w_off[j], (int)((unsigned)s * (BK * 2u)), 0, 0);
         }
     };
@@ -308,10 +322,10 @@ __global__ void __launch_bounds__(WM * WN * 64, (WM * WN) / 4) gemm_dma_kernel(c
     // fragment addresses: row (.. + l32), logical chunk 2 kk + h at position (2 kk + h) ^ ((l32 >> 1) & 7)
     const int sw = (l32 >> 1) & 7;
     const int a_row = (wm * (32 * TM) + l32) * (BK * 2);
-    const int w_row = BM * BK * 2 + (wn * (32 * TN) + l32) * (BK * 2);
+    const int w_row = TB * BK * 2 + (wn * (32 * TN) + l32) * (BK * 2);
     struct Frag { u32x4 a[TM], w[TN]; };
     auto read_frag = [&](Frag& f, int s, int kk) __attribute__((always_inline)) {
-        const unsigned char* st = smem + (s & 1) * DMA_STAGE_BYTES;
+        const unsigned char* st = smem + (s & 1) * STAGE_BYTES;
         const int pos = ((2 * kk + h) ^ sw) * 16;
 #pragma unroll
         for (int i = 0; i < TM; i++) f.a[i] = *reinterpret_cast<const u32x4*>(st + a_row + i * 32 * (BK * 2) + pos);
@@ -322,14 +336,16 @@ __global__ void __launch_bounds__(WM * WN * 64, (WM * WN) / 4) gemm_dma_kernel(c
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) acc[i][j] = mfma<F16>(f.a[i], f.w[j], acc[i][j]);
+            for (int j = 0; j < TN; j++) acc[i][j] = mfma<F16>(f.w[j], f.a[i], acc[i][j]);
     };
 
     fetch_slab(0);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's part of slab 0 is in LDS
     __syncthreads();
     for (int s = 0; s < nslab; s++) {
-        // slab s+1 into the other stage: its readers (iteration s-1) are behind the last barrier
+        // slab s+1 into the other stage: its readers (iteration s-1) are behind the last barrier.
+        // (Spreading these loads over the four steps measured 9 % slower here: the compiler
+        // then makes the fragment reads that follow each load wait for it.)
         if (s + 1 < nslab) fetch_slab(s + 1);
 #pragma unroll
         for (int kk = 0; kk < BK / 16; kk++) {
@@ -343,18 +359,166 @@ __global__ void __launch_bounds__(WM * WN * 64, (WM * WN) / 4) gemm_dma_kernel(c
     store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * (32 * TM), n0 + wn * (32 * TN), l32, h);
 }
 
-// Measured on the Klein projections: 4 x 2 waves (two per SIMD, 64 x 128 each) 1090-1220
-// TFLOP/s; 2 x 2 waves (one per SIMD, 128 x 128 each, fewer LDS reads) 960-1120.
+// ---------------------------------------------------------------------------
+// Four-wave build: one wave per SIMD, each owning 128 x 128 of C (256 accumulation
+// registers, 8 fragment reads per 16 MFMAs: a third fewer LDS bytes per MFMA than
+// the 8-wave builds). One wave per SIMD has no neighbour to hide its waits, so the
+// schedule leaves none: the fragments of the next 16-wide step are read under the
+// MFMAs of the current one, and the slab's one barrier sits after the THIRD of the
+// four steps: by then every fragment of the slab is in registers, so the barrier
+// both frees the slab's LDS stage for slab s + 2 (fetched at once, a whole slab
+// before it is needed) and makes slab s + 1 (fetched a slab ago) visible, whose
+// first fragments are then read under the MFMAs of the fourth step. Same 128-byte
+// swizzled rows and two 64 KB stages as the direct-to-LDS build above.
+template <bool F16, typename TC>
+__global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
+    constexpr int TM = 4, TN = 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int h = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int logical = logical_tile();
+    const int tiles_row = g.tiles_n * g.groups;
+    const int tm = logical / tiles_row;
+    int tn = logical - tm * tiles_row;
+    const int grp = tn / g.tiles_n;
+    tn -= grp * g.tiles_n;
+    const void* const wp = grp == 0 ? g.w : g.w_more[grp - 1];
+    void* const cp = grp == 0 ? g.c : g.c_more[grp - 1];
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const unsigned a_span = ((unsigned)(g.m - 1) * (unsigned)g.lda + (unsigned)g.k) * 2u;
+    const unsigned w_span = ((unsigned)(g.n - 1) * (unsigned)g.ldw + (unsigned)g.k) * 2u;
+    const u32x4 a_rsrc = make_rsrc_words(g.a, a_span);
+    const u32x4 w_rsrc = make_rsrc_words(wp, w_span);
+    const unsigned lds0 = lds_address(smem);
+    // wave w fills rows 64 w + 8 j + lane / 8 (j < 8) of the A slab and of the W slab
+    unsigned a_off[8], w_off[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int r = wave * 64 + j * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ ((r >> 1) & 7);
+        const int ar = min(m0 + r, g.m - 1); // rows past the edge re-read the last row; never stored
+        const int wr = min(n0 + r, g.n - 1);
+        a_off[j] = ((unsigned)ar * (unsigned)g.lda + (unsigned)(c * 8)) * 2u;
+        w_off[j] = ((unsigned)wr * (unsigned)g.ldw + (unsigned)(c * 8)) * 2u;
+    }
+    const int nslab = g.k / BK;
+    const unsigned fetch_lds = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)wave * (64 * BK * 2));
+    // slabs past the end re-fetch the last slab into a stage nobody reads any more
+    // the i-th (i < 16) of the loads that bring this wave's part of slab s in
+    auto fetch_one = [&](int s, int i) __attribute__((always_inline)) {
+        const unsigned uo = (unsigned)(s < nslab ? s : nslab - 1) * (BK * 2u);
+        const unsigned base = fetch_lds + (unsigned)(s & 1) * DMA_STAGE_BYTES;
+        const int j = i >> 1;
+        if ((i & 1) == 0) load_to_lds_16(a_rsrc, base + (unsigned)j * (8 * BK * 2), a_off[j], uo);
+        else load_to_lds_16(w_rsrc, base + BM * BK * 2 + (unsigned)j * (8 * BK * 2), w_off[j], uo);
+    };
+    auto fetch_slab = [&](int s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) fetch_one(s, i);
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    // fragment addresses in stage 0: row (.. + l32), logical chunk 2 kk + h (kk < 4)
+    const int sw = (l32 >> 1) & 7;
+    unsigned fa[4], fw[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) {
+        const unsigned pos = (unsigned)(((2 * kk + h) ^ sw) * 16);
+        fa[kk] = lds0 + (unsigned)((wm * 128 + l32) * (BK * 2)) + pos;
+        fw[kk] = lds0 + (unsigned)(BM * BK * 2 + (wn * 128 + l32) * (BK * 2)) + pos;
+    }
+    typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
+    struct Frag { u32x4 a[TM], w[TN]; };
+    // the r-th of the 8 reads of a fragment set
+    auto read_one = [&](Frag& f, unsigned stage_off, int kk, int r) __attribute__((always_inline)) {
+        if (r < 4) f.a[r] = *(lds_u32x4_t)(fa[kk] + stage_off + (unsigned)(r * 32 * (BK * 2)));
+        else f.w[r - 4] = *(lds_u32x4_t)(fw[kk] + stage_off + (unsigned)((r - 4) * 32 * (BK * 2)));
+    };
+    // 16 MFMAs on `cur`, the 8 reads of `nxt` spread under the first of them; fetch >= 0: one
+    // load of slab `fetch` per MFMA (a burst of 16 would hold the wave at the memory queue)
+    auto mfma_step = [&](const Frag& cur, Frag& nxt, unsigned nxt_stage_off, int nxt_kk, int fetch) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            if (fetch >= 0) fetch_one(fetch, t);
+            if (t < 8) read_one(nxt, nxt_stage_off, nxt_kk, t);
+            __builtin_amdgcn_s_setprio(1);
+            acc[t >> 2][t & 3] = mfma<F16>(cur.w[t & 3], cur.a[t >> 2], acc[t >> 2][t & 3]);
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    fetch_slab(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    __syncthreads();
+    fetch_slab(1);
+    Frag f0, f1;
+#pragma unroll
+    for (int r = 0; r < 8; r++) read_one(f0, 0u, 0, r);
+    for (int s = 0; s < nslab; s++) {
+        const unsigned so = (unsigned)(s & 1) * DMA_STAGE_BYTES;
+        const unsigned so_next = (unsigned)((s + 1) & 1) * DMA_STAGE_BYTES;
+        mfma_step(f0, f1, so, 1, -1);
+        mfma_step(f1, f0, so, 2, -1);
+        mfma_step(f0, f1, so, 3, -1);
+        // every fragment of slab s is in registers (lgkmcnt(0)) and this wave's part of slab
+        // s + 1 has landed (vmcnt(0)): behind the barrier slab s's stage is free and slab s + 1
+        // is visible
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        mfma_step(f1, f0, so_next, 0, s + 2);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
+    store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, l32, h);
+}
+
+// Measured on the Klein projections, same box: eight waves (two per SIMD, 64 x 128 each)
+// 1048-1217 TFLOP/s; four waves with the schedule above 1047-1248; four waves with the simple
+// loop of the eight-wave build 960-1120.
 constexpr int DMA_WM = 4, DMA_WN = 2;
 
+static int g_gemm_build = 1; // 256-tiles of 16-bit activations: 1 = four-wave build (default), 0 = eight-wave build (measurement knob)
+
+constexpr size_t kSmallLdsBytes = 2 * (size_t)(2 * 128 * BK * 2); // two stages of a 128-tile
+
 template <typename TA, bool F16, typename TC>
-static hipError_t launch_one(const GemmArgs& g, hipStream_t stream) {
-    const int64_t tiles_m = (g.m + BM - 1) / BM;
-    const int64_t nwg = tiles_m * g.tiles_n * g.groups;
+static hipError_t launch_one(const GemmArgs& g0, hipStream_t stream) {
+    GemmArgs g = g0;
+    const int64_t tiles256 = (int64_t)((g.m + 255) / 256) * ((g.n + 255) / 256) * g.groups;
+    if constexpr (!std::is_same<TA, float>::value) {
+        // fewer 256-tiles than five eighths of the CUs: 128-tiles, two workgroups per CU
+        if (g.k % BK == 0 && tiles256 < 160) {
+            g.tiles_n = (g.n + 127) / 128;
+            const int64_t nwg = (int64_t)((g.m + 127) / 128) * g.tiles_n * g.groups;
+            if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
+            gemm_dma_kernel<F16, TC, 2, 2, 128><<<dim3((unsigned)nwg), dim3(256), kSmallLdsBytes, stream>>>(g);
+            return hipGetLastError();
+        }
+    }
+    g.tiles_n = (g.n + BN - 1) / BN;
+    const int64_t nwg = tiles256;
     if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
     if constexpr (!std::is_same<TA, float>::value) {
+        if (g_gemm_build == 1 && g.k % BK == 0) {
+            gemm_ring_kernel<F16, TC><<<dim3((unsigned)nwg), dim3(256), kDmaLdsBytes, stream>>>(g);
+            return hipGetLastError();
+        }
         if (g.k % BK == 0) { // whole slabs of 16-bit activations: the direct-to-LDS build
-            gemm_dma_kernel<F16, TC, DMA_WM, DMA_WN><<<dim3((unsigned)nwg), dim3(DMA_WM * DMA_WN * 64), kDmaLdsBytes, stream>>>(g);
+            gemm_dma_kernel<F16, TC, DMA_WM, DMA_WN, 256><<<dim3((unsigned)nwg), dim3(DMA_WM * DMA_WN * 64), kDmaLdsBytes, stream>>>(g);
             return hipGetLastError();
         }
     }
@@ -365,8 +529,14 @@ static hipError_t launch_one(const GemmArgs& g, hipStream_t stream) {
 template <typename TA, bool F16, typename TC>
 static hipError_t raise_lds() {
     if constexpr (!std::is_same<TA, float>::value) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<F16, TC, DMA_WM, DMA_WN>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<F16, TC, DMA_WM, DMA_WN, 256>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLdsBytes);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<F16, TC, 2, 2, 128>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSmallLdsBytes);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_ring_kernel<F16, TC>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaLdsBytes);
         if (e != hipSuccess) return e;
     }
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<TA, F16, TC>),
@@ -394,6 +564,8 @@ hipError_t launch_gemm(const GemmArgs& g, int a_dtype, int w_dtype, int c_dtype,
     }
     return hipErrorInvalidValue;
 }
+
+void gemm_set_build(int build) { gemm::g_gemm_build = build == 1 ? 1 : 0; }
 
 hipError_t gemm_setup() {
     using namespace gemm;

@@ -26,5 +26,6 @@ int gemm_tile_cols();
 // a_dtype: kF32 or the weight's type; w_dtype: kF16 or kBF16; c_dtype: kF32 or the weight's type.
 hipError_t launch_gemm(const GemmArgs& args, int a_dtype, int w_dtype, int c_dtype, hipStream_t stream);
 hipError_t gemm_setup();
+void gemm_set_build(int build); // 256-tiles of 16-bit activations: 1 = four-wave build (default), 0 = eight-wave build
 
 } // namespace zdraw
