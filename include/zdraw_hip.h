@@ -341,6 +341,10 @@ int zdraw_hip_queue_sync(void* queue);
  * 1 = 4 waves x 32 query rows, two workgroups per CU. */
 void zdraw_hip_set_attention_variant(int variant);
 
+/* Measurement knob: which build multiplies 256 x 256 tiles of 16-bit activations.
+ * 1 = four waves, 128 x 128 each (default); 0 = eight waves, 64 x 128 each. */
+void zdraw_hip_set_gemm_build(int build);
+
 /* ABI drift guard (src/abi_gen.zig, runtime/abi_assert.zig:29): sizeof of the
  * shared structs as this library was compiled. which: 0 = ZdrawAttnParams,
  * 1 = ZdrawHipAttnExt, 2 = ZdrawHipQkOperands, 3 = ZdrawGemmParams,

@@ -311,3 +311,29 @@ def test_pair_and_triple_of_one_activation(ctx, pipe, count, same_shape):
         assert L.zdraw_hip_dispatch_count() == d0
     for b in [ab, wb] + cbs:
         b.release()
+
+
+@pytest.mark.parametrize("build", [1, 0])
+def test_many_tile_problem_runs_the_256_tile_builds(ctx, build):
+    # 13 x 13 = 169 tiles of 256 x 256 (ragged last row and column of tiles): enough tiles for
+    # the 256-tile builds (four waves by default, eight behind the knob), which the small
+    # shapes above never reach. Both against the oracle on identically rounded operands, and
+    # the two builds against each other at the same bar (their summation orders are the same
+    # per element, so in practice bit for bit).
+    L = hip.lib()
+    rng = np.random.default_rng(23)
+    m, k, n = 3300, 128, 3290
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
+    a_bits, ar = to16(a, hip.W_BF16)
+    w_bits, wr = to16(w, hip.W_BF16)
+    L.zdraw_hip_set_gemm_build(build)
+    try:
+        raw = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, hip.F32)
+    finally:
+        L.zdraw_hip_set_gemm_build(1)
+    got = raw.view(np.float32).reshape(m, n)
+    want = zo.linear_batch(ar, wr)
+    check(got, want, zo.linear_batch(a, w), k, a, w, f"169 tiles, build {build}")
+    # rows and columns of the ragged edge tiles
+    assert np.abs(got[-1] - want[-1]).max() < 1e-4 and np.abs(got[:, -1] - want[:, -1]).max() < 1e-4

@@ -1215,6 +1215,8 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
 
 void zdraw_hip_set_attention_variant(int variant) { g_variant = variant == 1 ? 1 : 0; }
 
+void zdraw_hip_set_gemm_build(int build) { gemm_set_build(build); }
+
 size_t zdraw_hip_abi_sizeof(int which) {
     switch (which) {
     case 0: return sizeof(ZdrawAttnParams);

@@ -136,6 +136,7 @@ SYMBOLS = {
     "zdraw_hip_event_release": (None, [_vp]),
     "zdraw_hip_queue_sync": (_int, [_vp]),
     "zdraw_hip_set_attention_variant": (None, [_int]),
+    "zdraw_hip_set_gemm_build": (None, [_int]),
     "zdraw_hip_abi_sizeof": (_sz, [_int]),
     "zdraw_hip_last_error": (C.c_char_p, []),
 }
