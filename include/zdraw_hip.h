@@ -336,9 +336,10 @@ float zdraw_hip_event_elapsed_ms(void* start, void* stop); /* negative on error 
 void zdraw_hip_event_release(void* event);
 int zdraw_hip_queue_sync(void* queue);
 
-/* Measurement knob: which build of the attention kernel runs.
+/* Measurement knob: which build of the attention kernel runs. Bit 0:
  * 0 = 8 waves x 32 query rows per workgroup, one workgroup per CU (default);
- * 1 = 4 waves x 32 query rows, two workgroups per CU. */
+ * 1 = 4 waves x 32 query rows, two workgroups per CU. Bit 1: 2 = never split the
+ * tiles of a thinly filled last round along the keys (by default they are). */
 void zdraw_hip_set_attention_variant(int variant);
 
 /* Measurement knob: which build multiplies 256 x 256 tiles of 16-bit activations.

@@ -404,16 +404,22 @@ def test_clock_probe_reports_every_workgroup_and_leaves_results_alone(ctx):
 
 
 def test_scratch_is_grow_only_and_filled(ctx):
+    # metal_api.m:6147-6191: a slot is (re)allocated only to grow, and a new allocation is
+    # filled before anyone reads it. The library uses the slots itself (pre-passed Q and K,
+    # key-split parts), so the test grows slot 4 past whatever it holds now.
     L = hip.lib()
-    a = L.zdraw_hip_attn_scratch(ctx.device, 4, 4096)
-    assert a and L.zdraw_hip_buffer_length(a) >= 4096
-    out = np.ones(4096, np.uint8)
-    L.zdraw_hip_read_buffer(a, out.ctypes.data_as(C.c_void_p), 4096)
+    cur = L.zdraw_hip_attn_scratch(ctx.device, 4, 16)
+    assert cur
+    want = 2 * L.zdraw_hip_buffer_length(cur) + 4096
+    a = L.zdraw_hip_attn_scratch(ctx.device, 4, want)
+    assert a and L.zdraw_hip_buffer_length(a) >= want
+    out = np.ones(want, np.uint8)
+    L.zdraw_hip_read_buffer(a, out.ctypes.data_as(C.c_void_p), want)
     assert not out.any()
     b = L.zdraw_hip_attn_scratch(ctx.device, 4, 1024)
-    assert b == a and L.zdraw_hip_buffer_length(b) >= 4096
-    c = L.zdraw_hip_attn_scratch(ctx.device, 4, 1 << 20)
-    assert L.zdraw_hip_buffer_length(c) >= (1 << 20)
+    assert b == a and L.zdraw_hip_buffer_length(b) >= want
+    c = L.zdraw_hip_attn_scratch(ctx.device, 4, want + (1 << 20))
+    assert L.zdraw_hip_buffer_length(c) >= want + (1 << 20)
     assert not L.zdraw_hip_attn_scratch(ctx.device, 5, 16)
 
 

@@ -139,13 +139,19 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 
     // XCD-aware remap: consecutive logical ids (one head's query blocks) share an XCD's L2
     int logical;
-    {
+    int split = 0;
+    if (a.splits > 1) {
+        // key-split tail: consecutive ids are the parts of one tile
+        const int t = (int)blockIdx.x / a.splits;
+        split = (int)blockIdx.x - t * a.splits;
+        logical = a.tile_base + t;
+    } else {
         const int nwg = gridDim.x;
         const int xcd = blockIdx.x & 7;
         const int idx = blockIdx.x >> 3;
         const int base = nwg >> 3;
         const int rem = nwg & 7;
-        logical = idx + xcd * base + (xcd < rem ? xcd : rem);
+        logical = a.tile_base + idx + xcd * base + (xcd < rem ? xcd : rem);
     }
     const int bh = logical / a.nqb;
     const int qb = logical - bh * a.nqb;
@@ -194,8 +200,15 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             nblk = __builtin_amdgcn_readfirstlane(s_nblocks);
         }
     }
+    // a key-split workgroup walks positions [i0, i0 + nblk) of the list
+    int i0 = 0;
+    if (a.splits > 1) {
+        const int per = (nblk + a.splits - 1) / a.splits;
+        i0 = split * per;
+        nblk = max(min(nblk - i0, per), 0);
+    }
     // wave-uniform by construction; readfirstlane lets the compiler keep it in scalar registers
-    auto block_of = [&](int i) -> int { return (MASKED && kp) ? __builtin_amdgcn_readfirstlane((int)blocks[i]) : i; };
+    auto block_of = [&](int i) -> int { return (MASKED && kp) ? __builtin_amdgcn_readfirstlane((int)blocks[i + i0]) : i + i0; };
 
     // ---- Q rows -> B-operand registers: qf[qi][s], lane: query 32*qi + l32, dims 16s + 8h .. +7
     // The workgroup's query rows are prepared in the layout that coalesces: 16 lanes per
@@ -749,7 +762,24 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         const float l_tot = pair_sum(l_run[qi]);
         const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         const int qrow = q0 + 32 * qi + l32;
-        if (qrow < a.tokens) {
+        if (a.splits > 1) {
+            // unnormalised rows, reference point and denominator of this part
+            const int64_t prow = ((int64_t)blockIdx.x * BQ + wave * QR + 32 * qi + l32);
+            float* op = a.part_o + prow * D;
+#pragma unroll
+            for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    f32x4 v;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j];
+                    *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
+                }
+            if (h == 0) {
+                a.part_ml[prow * 2] = BOUNDED ? 0.f : m_run[qi];
+                a.part_ml[prow * 2 + 1] = l_tot;
+            }
+        } else if (qrow < a.tokens) {
             const int64_t off = (int64_t)seg * a.o_bs + (int64_t)qrow * a.o_ts + (int64_t)head * a.o_hs;
             if (a.out_dtype == kF32) {
                 float* op = reinterpret_cast<float*>(a.o) + off;
@@ -794,13 +824,78 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     }
 }
 
+// Combines the parts of the key-split tiles: out[row] = sum_z O_z 2^(m_z - M) / sum_z l_z 2^(m_z - M),
+// M = max_z m_z, z ascending (m_z = -inf: an empty part, weight 0). 32 lanes per row, 4 dims each.
+__global__ void __launch_bounds__(256) attn_merge_kernel(const AttnArgs a, int block_rows) {
+    const int r = (int)blockIdx.x * 8 + (int)(threadIdx.x >> 5); // row among tail_tiles x block_rows
+    const int t = r / block_rows;
+    const int rr = r - t * block_rows;
+    const int logical = a.tile_base + t;
+    const int bh = logical / a.nqb;
+    const int qb = logical - bh * a.nqb;
+    const int seg = bh / a.heads;
+    const int head = bh - seg * a.heads;
+    const int qrow = qb * block_rows + rr;
+    if (qrow >= a.tokens) return;
+    const int d0 = (threadIdx.x & 31) * 4;
+    float M = -INFINITY;
+    for (int z = 0; z < a.splits; z++) {
+        const float* ml = a.part_ml + (((int64_t)t * a.splits + z) * block_rows + rr) * 2;
+        M = (ml[1] > 0.f) ? fmaxf(M, ml[0]) : M;
+    }
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    float l = 0.f;
+    for (int z = 0; z < a.splits; z++) {
+        const int64_t prow = ((int64_t)t * a.splits + z) * block_rows + rr;
+        const float* ml = a.part_ml + prow * 2;
+        if (!(ml[1] > 0.f)) continue; // a part that admitted no key
+        const float w = __builtin_amdgcn_exp2f(ml[0] - M);
+        l += ml[1] * w;
+        const f32x4 x = *reinterpret_cast<const f32x4*>(a.part_o + prow * D + d0);
+        acc += x * w;
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    acc *= inv;
+    const int64_t off = (int64_t)seg * a.o_bs + (int64_t)qrow * a.o_ts + (int64_t)head * a.o_hs + d0;
+    if (a.out_dtype == kF32) {
+        *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(a.o) + off) = acc;
+    } else if (a.out_dtype == kF16) {
+        typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<f16x4*>(reinterpret_cast<_Float16*>(a.o) + off) = __builtin_convertvector(acc, f16x4);
+    } else {
+        *reinterpret_cast<bf16x4*>(reinterpret_cast<bf16_t*>(a.o) + off) = __builtin_convertvector(acc, bf16x4);
+    }
+}
+
+// Whole tiles first, then (tail.splits > 1) the tiles of the last round in parts, then the merge.
 template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
-static hipError_t launch_one(const AttnArgs& a, hipStream_t stream) {
-    const int64_t nwg = (int64_t)a.nqb * a.heads * a.batch;
+static hipError_t launch_one(const AttnArgs& a0, hipStream_t stream) {
+    const int64_t nwg = (int64_t)a0.nqb * a0.heads * a0.batch;
     if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
-    attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
-        <<<dim3((unsigned)nwg), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
-    return hipGetLastError();
+    const int tail = a0.splits > 1 ? a0.tile_base : 0; // the planner leaves the tail size in tile_base
+    AttnArgs a = a0;
+    a.tile_base = 0;
+    a.splits = 1;
+    const int64_t whole = nwg - tail;
+    if (whole > 0) {
+        attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
+            <<<dim3((unsigned)whole), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (tail > 0) {
+        a.tile_base = (int32_t)whole;
+        a.splits = a0.splits;
+        a.clock_probe = nullptr;
+        attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
+            <<<dim3((unsigned)(tail * a0.splits)), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        const int rows = tail * NW * 32 * QB;
+        attn_merge_kernel<<<dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream>>>(a, NW * 32 * QB);
+        return hipGetLastError();
+    }
+    return hipSuccess;
 }
 
 template <typename TIn, bool MASKED, bool BOUNDED, int QB, int NW>
@@ -855,6 +950,28 @@ static hipError_t raise_shape() {
 } // namespace fwd
 
 int attention_block_rows(int shape) { return shape == 1 ? 128 : 256; }
+
+void attention_tail_plan(int64_t tiles, int cus, int key_blocks, int* tail_tiles, int* splits) {
+    *tail_tiles = 0;
+    *splits = 1;
+    if (tiles <= 0 || cus <= 0) return;
+    const int tail = (int)(tiles % cus);
+    // a last round that fills at most half the CUs: split its tiles along the keys so that it
+    // fills them all; each part keeps at least 8 key blocks
+    if (tail == 0 || tail * 2 > cus) return;
+    int s = cus / tail;
+    if (s > 16) s = 16;
+    if (s > key_blocks / 8) s = key_blocks / 8;
+    if (s < 2) return;
+    *tail_tiles = tail;
+    *splits = s;
+}
+size_t attention_part_o_bytes(int tail_tiles, int splits, int shape) {
+    return (size_t)tail_tiles * splits * attention_block_rows(shape) * D * sizeof(float);
+}
+size_t attention_part_ml_bytes(int tail_tiles, int splits, int shape) {
+    return (size_t)tail_tiles * splits * attention_block_rows(shape) * 2 * sizeof(float);
+}
 int attention_key_block() { return fwd::KB; }
 int attention_max_tokens() { return fwd::MAX_BLOCKS * fwd::KB; }
 

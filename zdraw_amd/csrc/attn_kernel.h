@@ -67,6 +67,13 @@ struct AttnArgs {
     // cycles at [2i] and as ticks of the fixed 100 MHz reference at [2i+1], i < clock_cap
     unsigned long long* clock_probe;
     int64_t clock_cap;
+    // Key-split launches (splits > 1): workgroup id = (tile - tile_base) * splits + z; split z
+    // walks the z-th part of the tile's key-block list and writes its unnormalised O^T rows,
+    // reference point and denominator; attn_merge_kernel combines them in z order.
+    int32_t tile_base;  // first logical tile (segment, head, query block) of this launch
+    int32_t splits;     // 0 or 1 = none
+    float* part_o;      // f32 [tile - tile_base][splits][block rows][128]
+    float* part_ml;     // f32 [tile - tile_base][splits][block rows][2]
 };
 
 // Standalone norm + rope over rows of one operand (Q or K): the pre-pass for
@@ -122,6 +129,13 @@ hipError_t wide_setup();
 // Launch one attention forward. in_dtype is kF32 or kBF16; k_mode is the
 // QkMode applied to K rows inside the K-block load. Returns a hipError_t.
 hipError_t launch_attention(const AttnArgs& args, int in_dtype, int k_mode, int shape, hipStream_t stream);
+// Tail plan for a launch of `tiles` workgroup tiles on `cus` compute units: how many tiles of
+// the last, partly filled round are better split along the keys, and into how many parts
+// (0 tiles = run everything whole). key_blocks = 32-key blocks per tile.
+void attention_tail_plan(int64_t tiles, int cus, int key_blocks, int* tail_tiles, int* splits);
+// Bytes of part_o and part_ml that `tail_tiles` x `splits` need for the kernel shape.
+size_t attention_part_o_bytes(int tail_tiles, int splits, int shape);
+size_t attention_part_ml_bytes(int tail_tiles, int splits, int shape);
 // Normalise + rotate `count` (1 or 2) operands of equal shape in one launch.
 hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipStream_t stream);
 // One-time per-device setup (raises the dynamic LDS limit on every instantiation).

@@ -36,6 +36,7 @@ namespace {
 
 struct Device {
     int ordinal;
+    int cus; // compute units: workgroup slots of the one-workgroup-per-CU kernels
 };
 struct Queue {
     Device* dev;
@@ -63,7 +64,7 @@ uint64_t g_dispatch = 0;
 uint64_t g_command = 0;
 uint64_t g_fallback = 0;
 uint64_t g_gpu_ns = 0;
-int g_variant = 0; // kernel shape: 0 = 8 waves per workgroup, 1 = 4 waves (two workgroups per CU)
+int g_variant = 0; // bit 0: kernel shape, 0 = 8 waves per workgroup, 1 = 4 waves (two workgroups per CU); bit 1: never split tail tiles
 bool g_setup_done = false;
 bool g_gemm_setup_done = false;
 
@@ -234,7 +235,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     a.heads = (int32_t)p->heads;
     a.batch = (int32_t)x->batch;
     a.key_limit = (int32_t)((p->valid != 0 && p->valid < p->tokens) ? p->valid : p->tokens);
-    const int rows = attention_block_rows(g_variant);
+    const int rows = attention_block_rows(g_variant & 1);
     a.nqb = (int32_t)((p->tokens + rows - 1) / rows);
     a.q_mode = (int32_t)x->qk_mode;
     a.out_dtype = (int32_t)x->out_dtype;
@@ -314,6 +315,25 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         a.mask_bs = (int64_t)x->mask_batch_bytes;
     }
 
+    // A last round of workgroups that fills at most half the CUs is split along the keys so
+    // that it fills them all (its parts are merged by a small kernel, in a fixed order).
+    if ((g_variant & 2) == 0) {
+        int tail = 0, splits = 1;
+        attention_tail_plan((int64_t)a.nqb * a.heads * a.batch, dev->cus, (a.key_limit + attention_key_block() - 1) / attention_key_block(),
+                            &tail, &splits);
+        if (splits > 1) {
+            Buffer* po = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 3, attention_part_o_bytes(tail, splits, g_variant & 1)));
+            Buffer* pm = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 4, attention_part_ml_bytes(tail, splits, g_variant & 1)));
+            if (!po || !pm) {
+                set_err("scratch allocation failed");
+                return ZDRAW_HIP_ERR_HANDLE;
+            }
+            a.splits = splits;
+            a.tile_base = tail; // launch_attention reads the tail size here
+            a.part_o = static_cast<float*>(po->ptr);
+            a.part_ml = static_cast<float*>(pm->ptr);
+        }
+    }
     plan->args = a;
     plan->in_dtype = (int)x->in_dtype;
     plan->k_mode = (int)x->qk_mode;
@@ -393,14 +413,15 @@ int enqueue(const FusedPlan& plan, hipStream_t stream) {
         if (g_clock_buf) {
             args.clock_probe = g_clock_buf;
             args.clock_cap = kClockCap;
-            g_clock_wgs = (int64_t)args.nqb * args.heads * args.batch;
+            // key-split tail tiles carry no probe
+            g_clock_wgs = (int64_t)args.nqb * args.heads * args.batch - (args.splits > 1 ? args.tile_base : 0);
             g_clock_stream = stream;
         }
     }
     TracePair tp{nullptr, nullptr};
     if (g_trace && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
         (void)hipEventRecord(tp.a, stream);
-    hipError_t e = launch_attention(args, plan.in_dtype, plan.k_mode, g_variant, stream);
+    hipError_t e = launch_attention(args, plan.in_dtype, plan.k_mode, g_variant & 1, stream);
     if (e != hipSuccess) {
         set_err("attention launch: %s", hipGetErrorString(e));
         return ZDRAW_HIP_ERR_HANDLE;
@@ -645,7 +666,7 @@ void* zdraw_hip_create_device(void) {
     // ZDRAW_ATTN_VARIANT picks the kernel build for a whole process (measurement aid)
     if (const char* v = getenv("ZDRAW_ATTN_VARIANT")) zdraw_hip_set_attention_variant(atoi(v));
     if (const char* v = getenv("ZDRAW_GEMM_BUILD")) gemm_set_build(atoi(v));
-    Device* d = new Device{0};
+    Device* d = new Device{0, prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256};
     return d;
 }
 
@@ -745,7 +766,7 @@ size_t zdraw_hip_pipeline_threads(void* pipeline) {
     Pipeline* p = static_cast<Pipeline*>(pipeline);
     if (!p) return 0;
     if (p->kind == 2 || p->kind == 3) return 512;
-    return p->kind == 0 ? (g_variant == 0 ? 512 : 256) : 256;
+    return p->kind == 0 ? ((g_variant & 1) == 0 ? 512 : 256) : 256;
 }
 
 // ---------------------------------------------------------------- attention
@@ -1213,7 +1234,7 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
     return m;
 }
 
-void zdraw_hip_set_attention_variant(int variant) { g_variant = variant == 1 ? 1 : 0; }
+void zdraw_hip_set_attention_variant(int variant) { g_variant = variant & 3; }
 
 void zdraw_hip_set_gemm_build(int build) { gemm_set_build(build); }
 
