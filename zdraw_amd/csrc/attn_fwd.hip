@@ -62,9 +62,14 @@ constexpr float kTau = 8.0f;             // log2 headroom of the lazy softmax ma
 // one), 4 stages when two workgroups share the CU's LDS (stored two steps
 // ahead, one barrier per step).
 constexpr int ring_stages(int qb, int nw) { return (qb == 2 || nw == 8) ? 8 : 4; }
+constexpr size_t kListBytes = (size_t)MAX_BLOCKS * (sizeof(unsigned short) + sizeof(unsigned));
 constexpr size_t lds_bytes(int nst) {
-    // ring + key-block list (u16) + per-block exclusion masks (u32)
-    return (size_t)nst * (KS_ELEMS + VS_ELEMS) * sizeof(bf16_t) + (size_t)MAX_BLOCKS * (sizeof(unsigned short) + sizeof(unsigned));
+    // ring + key-block list (u16) + per-block exclusion masks (u32); the 8-stage build also
+    // needs 24 KB behind the lists of its unpadded (direct-to-LDS) layout, where three waves
+    // park their query rows (the padded layout's ring is the larger one, short by 4 KB)
+    const size_t padded = (size_t)nst * (KS_ELEMS + VS_ELEMS) * sizeof(bf16_t) + kListBytes;
+    const size_t direct = (size_t)nst * 2 * (KB * D) * sizeof(bf16_t) + kListBytes + 3 * (size_t)(KB * D) * sizeof(bf16_t);
+    return nst == 8 && direct > padded ? direct : padded;
 }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -219,7 +224,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // own row from memory would touch one cache line per lane and instruction.
     // log2(e)/sqrt(D) rides on Q, so the MFMA delivers scores in the exp2 domain.
     bf16x8 qf[QB][8];
-    {
+    if constexpr (!DMA) {
         constexpr int QPITCH = D + 8;
         constexpr int RPP = NT / 16;      // rows per pass
         constexpr int PASSES = BQ / RPP;  // 8 QB
@@ -272,6 +277,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 qf[qi][s] = *reinterpret_cast<const bf16x8*>(Qs + (wave * QR + 32 * qi + l32) * QPITCH + 16 * s + 8 * h);
         __syncthreads(); // the ring may be filled from here on
     }
+    // (The direct-to-LDS build fetches its query rows together with the first K/V blocks, below.)
 
     // ---- block staging: thread t owns key t/TPK of the block, CPT chunks of 8 dims of K and of V
     const int lk_key = tid / TPK;
@@ -696,9 +702,32 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     if (nblk > 0) {
         // prologue: blocks 0 .. AHEAD-1 into the ring, blocks AHEAD and AHEAD+1 in flight
         if constexpr (DMA) {
+            // The wave's 32 prepared query rows (bf16, scale folded in) and the first AHEAD K/V
+            // blocks are requested together: one memory latency for all of it. Each wave parks
+            // its rows in 8 KB that the ring does not use yet (K stages 5-7, V stages 5-6, and
+            // the area behind the lists), in the K layout (chunk c of row r at c ^ (r & 15)),
+            // and is their only reader, so it needs no barrier for them, only its own vmcnt.
+            const unsigned q_span = ((unsigned)(a.tokens - 1) * (unsigned)a.q_ts + D) * 2u;
+            const u32x4 q_rsrc = make_rsrc_words(reinterpret_cast<const bf16_t*>(a.q) + (int64_t)seg * a.q_bs + (int64_t)head * a.q_hs, q_span);
+            const unsigned q_lds = __builtin_amdgcn_readfirstlane(
+                wave < 3   ? lds_address(Ks) + (unsigned)((5 + wave) * (KSTAGE * 2))
+                : wave < 5 ? lds_address(Vs) + (unsigned)((5 + wave - 3) * (VSTAGE * 2))
+                           : lds_address(Vs) + (unsigned)(NST * (VSTAGE * 2) + (int)kListBytes + (wave - 5) * (KB * D * 2)));
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int r = 4 * j + (lane >> 4);
+                const int qrow = min(q0 + r, a.tokens - 1); // rows past the sequence re-read the last row (never stored)
+                const unsigned off = ((unsigned)qrow * (unsigned)a.q_ts + (unsigned)(((lane & 15) ^ (r & 15)) * 8)) * 2u;
+                load_to_lds_16(q_rsrc, q_lds + (unsigned)(j * 1024), off, 0u);
+            }
 #pragma unroll
             for (int i = 0; i < AHEAD; i++) dma_fetch(i, i);
             __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+            asm volatile("" ::: "memory");
+            typedef const __attribute__((address_space(3))) bf16x8* lds_q_t;
+#pragma unroll
+            for (int s = 0; s < 8; s++)
+                qf[0][s] = *(lds_q_t)(q_lds + (unsigned)(l32 * (D * 2) + (((2 * s + h) ^ (l32 & 15)) * 16)));
         } else {
             StageRegs pre[AHEAD];
 #pragma unroll
@@ -779,10 +808,9 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 a.part_ml[prow * 2] = BOUNDED ? 0.f : m_run[qi];
                 a.part_ml[prow * 2 + 1] = l_tot;
             }
-        } else if (qrow < a.tokens) {
-            const int64_t off = (int64_t)seg * a.o_bs + (int64_t)qrow * a.o_ts + (int64_t)head * a.o_hs;
-            if (a.out_dtype == kF32) {
-                float* op = reinterpret_cast<float*>(a.o) + off;
+        } else if (a.out_dtype == kF32) {
+            if (qrow < a.tokens) {
+                float* op = reinterpret_cast<float*>(a.o) + (int64_t)seg * a.o_bs + (int64_t)qrow * a.o_ts + (int64_t)head * a.o_hs;
 #pragma unroll
                 for (int blk = 0; blk < 4; blk++)
 #pragma unroll
@@ -792,29 +820,37 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                         for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
                         *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
                     }
-            } else if (a.out_dtype == kF16) {
-                typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-                _Float16* op = reinterpret_cast<_Float16*>(a.o) + off;
+            }
+        } else {
+            // 16-bit output: a lane holds one row in 8-byte pieces, which would leave the chip as
+            // 32 sixteen-byte segments per store instruction. The wave turns its 32 x 128 tile
+            // through 8 KB of LDS (its own stage of the idle K ring, K layout: chunk c of row r
+            // at c ^ (r & 15)) and stores whole 256-byte rows, four per instruction.
+            __syncthreads(); // every wave is done with the ring
+            typedef __attribute__((address_space(3))) u32x2* lds_u32x2_t;
+            typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
+            typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+            const unsigned o_lds = lds_address(Ks) + (unsigned)((wave * QB + qi) * (KSTAGE * 2));
+            const bool half = a.out_dtype == kF16;
 #pragma unroll
-                for (int blk = 0; blk < 4; blk++)
+            for (int blk = 0; blk < 4; blk++)
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        f32x4 v;
+                for (int i = 0; i < 4; i++) {
+                    f32x4 v;
 #pragma unroll
-                        for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
-                        *reinterpret_cast<f16x4*>(op + 32 * blk + 8 * i + 4 * h) = __builtin_convertvector(v, f16x4);
-                    }
-            } else {
-                bf16_t* op = reinterpret_cast<bf16_t*>(a.o) + off;
+                    for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
+                    const u32x2 bits = half ? __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4))
+                                            : __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
+                    *(lds_u32x2_t)(o_lds + (unsigned)(l32 * (D * 2) + (((4 * blk + i) ^ (l32 & 15)) * 16) + 8 * h)) = bits;
+                }
+            unsigned short* const obase = reinterpret_cast<unsigned short*>(a.o) + (int64_t)seg * a.o_bs + (int64_t)head * a.o_hs;
 #pragma unroll
-                for (int blk = 0; blk < 4; blk++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        f32x4 v;
-#pragma unroll
-                        for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
-                        *reinterpret_cast<bf16x4*>(op + 32 * blk + 8 * i + 4 * h) = __builtin_convertvector(v, bf16x4);
-                    }
+            for (int j = 0; j < 8; j++) {
+                const int r = 4 * j + (lane >> 4);
+                const u32x4 row16 = *(lds_u32x4_t)(o_lds + (unsigned)(r * (D * 2) + (lane & 15) * 16));
+                const int orow = q0 + 32 * qi + r;
+                if (orow < a.tokens)
+                    *reinterpret_cast<u32x4*>(obase + (int64_t)orow * a.o_ts + (((lane & 15) ^ (r & 15)) * 8)) = row16;
             }
         }
     }
@@ -910,6 +946,8 @@ static hipError_t launch_kmode(const AttnArgs& a, int k_mode, hipStream_t stream
 
 template <typename TIn, int QB, int NW>
 static hipError_t launch_flags(const AttnArgs& a, int k_mode, hipStream_t stream) {
+    // Q and K are prepared at the same site: the builds rely on it
+    if ((k_mode == kQkNone) != (a.q_mode == kQkNone)) return hipErrorInvalidValue;
     // the masked build is only needed when some key of some block is excluded
     const bool masked = a.key_pad != nullptr || (a.key_limit % KB) != 0;
     const bool bounded = a.bounded != 0;
