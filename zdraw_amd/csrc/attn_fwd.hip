@@ -385,7 +385,8 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // LDS byte addresses of this wave's four rows in stage 0 of the K ring and of the V ring
     const unsigned dma_k_lds = __builtin_amdgcn_readfirstlane(lds_address(Ks) + (unsigned)(4 * wave * D * 2));
     const unsigned dma_v_lds = __builtin_amdgcn_readfirstlane(lds_address(Vs) + (unsigned)(4 * wave * D * 2));
-    auto dma_fetch = [&](int i, int stage) __attribute__((always_inline)) {
+    // which: 1 = the K block, 2 = the V block, 3 = both
+    auto dma_fetch_part = [&](int i, int stage, int which) __attribute__((always_inline)) {
         const int ii = i < nblk ? i : nblk - 1; // past the end: a harmless re-fetch into a dead stage
         const int blk = block_of(ii);
         unsigned ko = dma_k_off, vo = dma_v_off;
@@ -394,9 +395,10 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             ko = tail ? dma_k_off_tail : dma_k_off;
             vo = tail ? dma_v_off_tail : dma_v_off;
         }
-        load_to_lds_16(dma_k_rsrc, dma_k_lds + (unsigned)stage * (KSTAGE * 2u), ko, (unsigned)blk * k_blk_bytes);
-        load_to_lds_16(dma_v_rsrc, dma_v_lds + (unsigned)stage * (VSTAGE * 2u), vo, (unsigned)blk * v_blk_bytes);
+        if (which & 1) load_to_lds_16(dma_k_rsrc, dma_k_lds + (unsigned)stage * (KSTAGE * 2u), ko, (unsigned)blk * k_blk_bytes);
+        if (which & 2) load_to_lds_16(dma_v_rsrc, dma_v_lds + (unsigned)stage * (VSTAGE * 2u), vo, (unsigned)blk * v_blk_bytes);
     };
+    auto dma_fetch = [&](int i, int stage) __attribute__((always_inline)) { dma_fetch_part(i, stage, 3); };
 
     // ---- running state
     f32x16 oacc[QB][4]; // O^T: lane query 32*qi + l32, dims 32*blk + 8i + 4h + j
@@ -720,9 +722,20 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 const unsigned off = ((unsigned)qrow * (unsigned)a.q_ts + (unsigned)(((lane & 15) ^ (r & 15)) * 8)) * 2u;
                 load_to_lds_16(q_rsrc, q_lds + (unsigned)(j * 1024), off, 0u);
             }
-#pragma unroll
-            for (int i = 0; i < AHEAD; i++) dma_fetch(i, i);
-            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+            // what the first two steps read before their barrier (K blocks 0..3, V blocks 0 and 1:
+            // step 1 already reads the first fragments of step 2) is requested first and waited
+            // for here; the rest of the first AHEAD blocks (4 loads) is covered by the wait before
+            // the barrier that ends step 1. Every workgroup of a round starts at once, so these
+            // first loads arrive at the rate of memory, not at its latency.
+            static_assert(AHEAD == 5, "the prologue's load count assumes five blocks ahead");
+            dma_fetch_part(0, 0, 3);
+            dma_fetch_part(1, 1, 3);
+            dma_fetch_part(2, 2, 1);
+            dma_fetch_part(3, 3, 1);
+            dma_fetch_part(2, 2, 2);
+            dma_fetch_part(3, 3, 2);
+            dma_fetch_part(4, 4, 3);
+            __builtin_amdgcn_s_waitcnt(0x0F74); // vmcnt(4)
             asm volatile("" ::: "memory");
             typedef const __attribute__((address_space(3))) bf16x8* lds_q_t;
 #pragma unroll
