@@ -313,27 +313,40 @@ def test_pair_and_triple_of_one_activation(ctx, pipe, count, same_shape):
         b.release()
 
 
+@pytest.mark.parametrize("c_dtype", [hip.F32, hip.BF16])
 @pytest.mark.parametrize("build", [1, 0])
-def test_many_tile_problem_runs_the_256_tile_builds(ctx, build):
+def test_many_tile_problem_runs_the_256_tile_builds(ctx, build, c_dtype):
     # 13 x 13 = 169 tiles of 256 x 256 (ragged last row and column of tiles): enough tiles for
     # the 256-tile builds (four waves by default, eight behind the knob), which the small
-    # shapes above never reach. Both against the oracle on identically rounded operands, and
-    # the two builds against each other at the same bar (their summation orders are the same
-    # per element, so in practice bit for bit).
+    # shapes above never reach; with 16-bit C the interior tiles leave through LDS as whole
+    # rows and the edge tiles element by element. Against the oracle on identically rounded
+    # operands.
     L = hip.lib()
     rng = np.random.default_rng(23)
     m, k, n = 3300, 128, 3290
+    ldc = 3296  # rows of C start 16-byte aligned
     a = rng.standard_normal((m, k), dtype=np.float32)
     w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
     a_bits, ar = to16(a, hip.W_BF16)
     w_bits, wr = to16(w, hip.W_BF16)
     L.zdraw_hip_set_gemm_build(build)
     try:
-        raw = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, hip.F32)
+        raw = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, c_dtype, ldc=ldc,
+                      c_init=np.zeros(m * ldc * (4 if c_dtype == hip.F32 else 2), np.uint8))
     finally:
         L.zdraw_hip_set_gemm_build(1)
-    got = raw.view(np.float32).reshape(m, n)
     want = zo.linear_batch(ar, wr)
-    check(got, want, zo.linear_batch(a, w), k, a, w, f"169 tiles, build {build}")
+    if c_dtype == hip.F32:
+        got = raw.view(np.float32).reshape(m, ldc)[:, :n]
+        check(got, want, zo.linear_batch(a, w), k, a, w, f"169 tiles, build {build}")
+        tol = 1e-4
+    else:
+        full = raw.view(np.uint16).reshape(m, ldc)
+        got = from16(full[:, :n], hip.W_BF16)
+        assert not full[:, n:].any()  # the pad columns of the pitch stay untouched
+        s = np.sqrt(k) * np.sqrt(np.mean(ar.astype(np.float64) ** 2)) * np.sqrt(np.mean(wr.astype(np.float64) ** 2))
+        err = np.abs(got - want)
+        assert err.max() <= 2 ** -8 * np.abs(want).max() + 2e-5 * s  # one bf16 rounding of the fp32 result
+        tol = 2 ** -8 * np.abs(want).max() + 1e-4
     # rows and columns of the ragged edge tiles
-    assert np.abs(got[-1] - want[-1]).max() < 1e-4 and np.abs(got[:, -1] - want[:, -1]).max() < 1e-4
+    assert np.abs(got[-1] - want[-1]).max() < tol and np.abs(got[:, -1] - want[:, -1]).max() < tol
