@@ -342,6 +342,14 @@ int zdraw_hip_queue_sync(void* queue);
  * tiles of a thinly filled last round along the keys (by default they are). */
 void zdraw_hip_set_attention_variant(int variant);
 
+/* How a launch of `tiles` workgroup tiles (segments x heads x query blocks) is laid on `cus`
+ * compute units (no reference counterpart: scheduling, exposed so that it can be checked
+ * without a device). A last round that fills at most half the CUs is split along the keys:
+ * *tail_tiles tiles (the last ones) run as *splits parts each, at least 8 key blocks per part,
+ * at most 16 parts; *tail_tiles = 0 and *splits = 1 when everything runs whole. */
+void zdraw_hip_attention_tail_plan(uint64_t tiles, uint32_t cus, uint32_t key_blocks, uint32_t* tail_tiles,
+                                   uint32_t* splits);
+
 /* Measurement knob: which build multiplies 256 x 256 tiles of 16-bit activations.
  * 1 = four waves, 128 x 128 each (default); 0 = eight waves, 64 x 128 each. */
 void zdraw_hip_set_gemm_build(int build);

@@ -59,6 +59,31 @@ def test_abi_struct_sizes():
     assert "#define ZDRAW_HIP_ABI_GEMM_EXT_SIZE 48" in text
 
 
+def test_tail_plan_of_the_baseline_shapes():
+    # 256 CUs, one 256-row tile per workgroup: which last rounds are split along the keys
+    L = hip.lib()
+
+    def plan(tiles, key_blocks, cus=256):
+        t, s = C.c_uint32(99), C.c_uint32(99)
+        L.zdraw_hip_attention_tail_plan(tiles, cus, key_blocks, C.byref(t), C.byref(s))
+        return t.value, s.value
+
+    assert plan(18 * 24, 144) == (0, 1)        # Klein 1024^2: 432 tiles, a tail of 176 stays whole
+    assert plan(18 * 30, 144) == (28, 9)       # Z-Image 1024^2: 540 tiles = 2 rounds + 28
+    assert plan(6 * 24 * 4, 48) == (64, 4)     # Klein 512^2 x 4: 576 tiles = 2 rounds + 64
+    assert plan(34 * 24 * 2, 272) == (96, 2)   # ragged edit: 1632 tiles = 6 rounds + 96
+    assert plan(512, 144) == (0, 1)            # whole rounds
+    assert plan(6, 10) == (0, 1)               # too few key blocks to split (8 per part)
+    assert plan(6, 64) == (6, 8)               # a small launch spreads over the chip, 8 blocks per part
+    assert plan(2, 1024) == (2, 16)            # never more than 16 parts
+    assert plan(129, 144) == (0, 1)            # a tail above half the CUs stays whole
+    assert plan(128, 144) == (128, 2)
+    assert plan(0, 144) == (0, 1) and plan(10, 144, cus=0) == (0, 1)
+    for tiles in range(1, 700, 7):             # invariants
+        t, s = plan(tiles, 144)
+        assert (t == 0 and s == 1) or (t == tiles % 256 and 2 <= s <= 16 and t * s <= 256 and 144 // s >= 8)
+
+
 def test_pipeline_lookup_without_device_is_null():
     L = hip.lib()
     err = C.create_string_buffer(128)

@@ -1238,6 +1238,15 @@ void zdraw_hip_set_attention_variant(int variant) { g_variant = variant & 3; }
 
 void zdraw_hip_set_gemm_build(int build) { gemm_set_build(build); }
 
+void zdraw_hip_attention_tail_plan(uint64_t tiles, uint32_t cus, uint32_t key_blocks, uint32_t* tail_tiles,
+                                   uint32_t* splits) {
+    int t = 0, s = 1;
+    if (tiles <= 0x7fffffffull && cus <= 0x7fffffffu && key_blocks <= 0x7fffffffu)
+        attention_tail_plan((int64_t)tiles, (int)cus, (int)key_blocks, &t, &s);
+    if (tail_tiles) *tail_tiles = (uint32_t)t;
+    if (splits) *splits = (uint32_t)s;
+}
+
 size_t zdraw_hip_abi_sizeof(int which) {
     switch (which) {
     case 0: return sizeof(ZdrawAttnParams);

@@ -137,6 +137,7 @@ SYMBOLS = {
     "zdraw_hip_queue_sync": (_int, [_vp]),
     "zdraw_hip_set_attention_variant": (None, [_int]),
     "zdraw_hip_set_gemm_build": (None, [_int]),
+    "zdraw_hip_attention_tail_plan": (None, [_u64, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "zdraw_hip_abi_sizeof": (_sz, [_int]),
     "zdraw_hip_last_error": (C.c_char_p, []),
 }
