@@ -145,6 +145,19 @@ def test_matches_torch_sdpa_fp64(tokens, heads, kv, dim, causal):
     assert np.abs(got - want).max() < 2e-5
 
 
+def test_matches_committed_sdpa_fixtures():
+    # tests/golden/sdpa_fp64.npz (written by tests/golden/make_sdpa_fixtures.py): the same
+    # library cross-check as above on fixed inputs, without torch at hand
+    import os
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sdpa_fp64.npz"))
+    n = sum(1 for name in z.files if name.startswith("shape"))
+    assert n >= 7
+    for i in range(n):
+        tokens, heads, kv, dim, causal = (int(x) for x in z[f"shape{i}"])
+        got = zo.attention_run(z[f"q{i}"], z[f"k{i}"], z[f"v{i}"], cfg(tokens, heads, kv, dim, bool(causal)))
+        assert np.abs(got - z[f"o{i}"]).max() < 2e-5, (i, tokens, heads, kv, dim, causal)
+
+
 def test_valid_limit_matches_brute_force():
     rng = np.random.default_rng(3)
     c = cfg(50, 2, 2, 16, valid=37)
