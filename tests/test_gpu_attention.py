@@ -5,6 +5,7 @@ Tolerance of the bf16 path against the fp32 reference: max abs <= 2e-2 and
 mean abs <= 2e-3 (tests/refimpl.py). Run-to-run results must be bit-identical.
 """
 import ctypes as C
+import os
 import sys
 
 import numpy as np
@@ -65,6 +66,25 @@ def test_tiny_reference_case_takes_the_fallback_contract(ctx):
     assert np.allclose(got, want, atol=1e-4)
     with pytest.raises(host.UnsupportedShape):
         host.attention_fast_run(ctx, q, q, v, cfg, cpu=None)
+
+
+def test_committed_sdpa_fixtures(ctx):
+    # tests/golden/sdpa_fp64.npz: a library's fp64 results on fixed inputs; the shapes this
+    # backend runs (head_dim 128, one K/V head per head, not causal) at the bf16 bar, the
+    # others refused
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sdpa_fp64.npz"))
+    ran = 0
+    for i in range(sum(1 for name in z.files if name.startswith("shape"))):
+        tokens, heads, kv, dim, causal = (int(x) for x in z[f"shape{i}"])
+        cfg = host.Config(tokens, heads, kv, dim, bool(causal))
+        if dim == 128 and kv == heads and not causal:
+            got = ctx.run(z[f"q{i}"], z[f"k{i}"], z[f"v{i}"], cfg)
+            refimpl.check_close(got, z[f"o{i}"], f"fixture {i}")
+            ran += 1
+        else:
+            with pytest.raises(host.UnsupportedShape):
+                ctx.run(z[f"q{i}"], z[f"k{i}"], z[f"v{i}"], cfg)
+    assert ran >= 3
 
 
 # metal/mattn_test.zig:47-53 (block_cases): D=128, tails inside and across tiles
