@@ -894,14 +894,25 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnArgs a, int b
     }
     f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
     float l = 0.f;
-    for (int z = 0; z < a.splits; z++) {
-        const int64_t prow = ((int64_t)t * a.splits + z) * block_rows + rr;
-        const float* ml = a.part_ml + prow * 2;
-        if (!(ml[1] > 0.f)) continue; // a part that admitted no key
-        const float w = __builtin_amdgcn_exp2f(ml[0] - M);
-        l += ml[1] * w;
-        const f32x4 x = *reinterpret_cast<const f32x4*>(a.part_o + prow * D + d0);
-        acc += x * w;
+    // four parts' loads in flight at a time; parts are still added in ascending order
+    for (int z0 = 0; z0 < a.splits; z0 += 4) {
+        f32x4 x[4];
+        float mz[4], lz[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int z = min(z0 + i, a.splits - 1);
+            const int64_t prow = ((int64_t)t * a.splits + z) * block_rows + rr;
+            mz[i] = a.part_ml[prow * 2];
+            lz[i] = z0 + i < a.splits ? a.part_ml[prow * 2 + 1] : 0.f;
+            x[i] = *reinterpret_cast<const f32x4*>(a.part_o + prow * D + d0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (!(lz[i] > 0.f)) continue; // past the last part, or a part that admitted no key
+            const float w = __builtin_amdgcn_exp2f(mz[i] - M);
+            l += lz[i] * w;
+            acc += x[i] * w;
+        }
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     acc *= inv;

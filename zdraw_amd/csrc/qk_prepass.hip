@@ -18,11 +18,11 @@ namespace zdraw {
 // in-place f32 token-major form. A lane reads and writes only its own 8
 // elements, so the output may alias the input.
 constexpr int kPrepTokens = 4; // tokens (waves) per workgroup
-constexpr int kPrepGroups = 6; // groups of four heads walked by one lane
 
-template <typename TIn, int MODE>
+// G = groups of four heads walked by one lane: 6 (24 heads per pass: Klein) or 8 (32 heads
+// per pass: Z-Image's 30 heads in one pass instead of two)
+template <typename TIn, int MODE, int G>
 __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const PrepPair pair) {
-    constexpr int G = kPrepGroups;
     // grid z = operand * batch + segment; the choice is uniform over the workgroup
     const int op = (int)blockIdx.z >= pair.op[0].batch ? 1 : 0;
     const PrepArgs& p = pair.op[op];
@@ -107,20 +107,28 @@ hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipSt
     PrepPair pair;
     pair.op[0] = ops[0];
     pair.op[1] = ops[count - 1];
-    const dim3 grid((unsigned)((p.tokens + kPrepTokens - 1) / kPrepTokens),
-                    (unsigned)((p.heads + 4 * kPrepGroups - 1) / (4 * kPrepGroups)), (unsigned)(p.batch * count));
+    const bool wide_pass = (p.heads + 31) / 32 < (p.heads + 23) / 24; // fewer passes over the heads with 32 per pass
+    const int per_pass = wide_pass ? 32 : 24;
+    const dim3 grid((unsigned)((p.tokens + kPrepTokens - 1) / kPrepTokens), (unsigned)((p.heads + per_pass - 1) / per_pass),
+                    (unsigned)(p.batch * count));
     const dim3 block(kPrepTokens * 64);
     const bool klein = p.mode == kQkKlein;
     if (!klein && p.mode != kQkZimage) return hipErrorInvalidValue;
+#define ZD_PREP(T, M) \
+    do { \
+        if (wide_pass) qk_prepass_kernel<T, M, 8><<<grid, block, 0, stream>>>(pair); \
+        else qk_prepass_kernel<T, M, 6><<<grid, block, 0, stream>>>(pair); \
+    } while (0)
     if (in_dtype == kF32) {
-        if (klein) qk_prepass_kernel<float, kQkKlein><<<grid, block, 0, stream>>>(pair);
-        else qk_prepass_kernel<float, kQkZimage><<<grid, block, 0, stream>>>(pair);
+        if (klein) ZD_PREP(float, kQkKlein);
+        else ZD_PREP(float, kQkZimage);
     } else if (in_dtype == kBF16) {
-        if (klein) qk_prepass_kernel<bf16_t, kQkKlein><<<grid, block, 0, stream>>>(pair);
-        else qk_prepass_kernel<bf16_t, kQkZimage><<<grid, block, 0, stream>>>(pair);
+        if (klein) ZD_PREP(bf16_t, kQkKlein);
+        else ZD_PREP(bf16_t, kQkZimage);
     } else {
         return hipErrorInvalidValue;
     }
+#undef ZD_PREP
     return hipGetLastError();
 }
 
