@@ -470,3 +470,51 @@ def test_qk_norm_rope_in_place_matches_oracle(ctx):
                    kv_heads=heads, head_dim=128, norm_eps=wl.ZIMAGE_EPS)
     qb.release()
     kb.release()
+
+
+# ------------------------------------------------ key-split tail tiles and their merge
+@pytest.mark.parametrize("tokens,valid,heads,bounded", [(700, 0, 2, True), (700, 650, 2, False), (1000, 0, 1, False),
+                                                       (1500, 1300, 3, True)])
+def test_key_split_tail_matches_whole_tiles_and_oracle(ctx, tokens, valid, heads, bounded):
+    # A launch far smaller than the chip is all tail: its tiles are split along the keys
+    # (at least 8 key blocks per part) and merged. Shapes with a ragged last block, a key
+    # limit, and both softmax forms; compared with the same call made whole (knob 2) and
+    # with the oracle on every row.
+    L = hip.lib()
+    rng = np.random.default_rng(tokens + heads)
+    shape = (tokens, heads, 128)
+    scale = 0.35 if bounded else 1.0
+    q, k, v = (rng.standard_normal(shape, dtype=np.float32) * np.float32(scale) for _ in range(3))
+    tail, splits = C.c_uint32(0), C.c_uint32(0)
+    key_blocks = ((valid or tokens) + 31) // 32
+    L.zdraw_hip_attention_tail_plan(((tokens + 255) // 256) * heads, 256, key_blocks, C.byref(tail), C.byref(splits))
+    assert splits.value >= 2 and tail.value == ((tokens + 255) // 256) * heads  # this test is about the split path
+    bufs = [ctx.buffer(host.f32_to_bf16_bits(a)) for a in (q, k, v)]
+    outs = []
+    for knob in (0, 2):
+        L.zdraw_hip_set_attention_variant(knob)
+        o = ctx.buffer(nbytes=q.size * 4)
+        p = hip.AttnParams(tokens, heads, heads, 128, 0, valid)
+        x = hip.AttnExt()
+        for s_ in (x.q_stride, x.k_stride, x.v_stride, x.out_stride):
+            s_[0], s_[1], s_[2] = 0, heads * 128, 128
+        x.batch, x.in_dtype, x.out_dtype, x.qk_mode = 1, hip.BF16, hip.F32, hip.QK_NONE
+        # |q.k|/sqrt(128) stays below 44 for these draws only in the scaled-down case
+        x.score_bound = 40.0 if bounded else 0.0
+        try:
+            rc = L.zdraw_hip_run_attention_fused(ctx.queue, bufs[0].handle, bufs[1].handle, bufs[2].handle, o.handle,
+                                                 C.byref(p), C.byref(x), None)
+        finally:
+            L.zdraw_hip_set_attention_variant(0)
+        assert rc == 0, hip.last_error()
+        outs.append(o.read(np.float32, shape))
+        o.release()
+    split, whole = outs
+    rb = lambda a: host.bf16_bits_to_f32(host.f32_to_bf16_bits(a))
+    want = zo.attention_run(rb(q), rb(k), rb(v), zo.Config(tokens, heads, heads, 128, False, valid))
+    refimpl.check_close(split, want, "key-split")
+    refimpl.check_close(whole, want, "whole")
+    # the two differ only in where the partial sums are cut: far below the bf16 bar
+    assert np.abs(split - whole).max() < 2e-3
+    for b in bufs:
+        b.release()

@@ -741,6 +741,16 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
             for (int s = 0; s < 8; s++)
                 qf[0][s] = *(lds_q_t)(q_lds + (unsigned)(l32 * (D * 2) + (((2 * s + h) ^ (l32 & 15)) * 16)));
+            // rows that did not pass the pre-pass (operands used as given) still need the softmax
+            // scale that the exp2-domain scores ride on (wave-uniform branch)
+            if (a.scale_log2 != 1.0f) {
+#pragma unroll
+                for (int s = 0; s < 8; s++) {
+                    f32x8 x = __builtin_convertvector(qf[0][s], f32x8);
+                    x *= a.scale_log2;
+                    qf[0][s] = __builtin_convertvector(x, bf16x8);
+                }
+            }
         } else {
             StageRegs pre[AHEAD];
 #pragma unroll
