@@ -11,19 +11,26 @@
 //     so every lane owns one query column: softmax reductions are in-lane plus
 //     one permlane32 swap, and the exponentiated block is already the B operand
 //     of the second MFMA (O^T = V^T . P^T): no LDS round trip for P;
-//   * K blocks sit in LDS row-major (272-byte pitch, conflict-free b128 reads);
-//     V blocks sit row-major too (320-byte pitch) and the V^T operand is built
-//     by the transposing LDS read ds_read_b64_tr_b16, so staging V is a plain copy;
-//   * RMSNorm + rope are applied to the Q rows once in the prologue and to the
-//     K rows between the global load and the LDS store of each block;
+//   * K and V blocks sit in LDS row-major; the V^T operand is built by the
+//     transposing LDS read ds_read_b64_tr_b16, so staging V is a plain copy;
+//   * Q and K normally arrive prepared (norm, rope, softmax scale: one pre-pass
+//     kernel per call) as bf16, and then query rows and K/V blocks go from global
+//     memory straight into LDS (buffer_load ... lds) in a swizzled, unpadded
+//     layout; otherwise RMSNorm + rope are applied to the Q rows in the prologue
+//     and to the K rows between the global load and the LDS store of each block
+//     (registers, padded rows);
 //   * keys are walked in blocks of 32 through an LDS ring; inside one wave the
 //     MFMAs of S(b+1) = K(b+1) Q^T and O += V(b-1)^T P(b-1) are interleaved, slot
 //     by slot, with the softmax VALU work of block b (the three are independent);
-//   * K/V blocks are fetched with buffer loads (descriptor + scalar block offset,
-//     no per-step address arithmetic) two steps ahead of the LDS store that
-//     consumes them; LDS fragment reads run ahead across step boundaries;
-//   * block order is fixed and nothing is accumulated with atomics, so the
-//     output is bit-identical from run to run.
+//   * blocks are requested five steps ahead (descriptor + scalar block offset, no
+//     per-step address arithmetic); LDS fragment reads run ahead across step
+//     boundaries; the main loop takes a whole turn of the ring per trip, so every
+//     LDS address in it is a register plus an immediate;
+//   * 16-bit outputs are turned through LDS and stored as whole rows; the tiles of
+//     a thinly filled last round of workgroups are split along the keys and merged
+//     by a small kernel in a fixed order;
+//   * block order and merge order are fixed and nothing is accumulated with
+//     atomics, so the output is bit-identical from run to run.
 #include "attn_device.hpp"
 
 namespace zdraw {
