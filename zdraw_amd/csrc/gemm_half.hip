@@ -9,17 +9,19 @@
 // contiguous in k), which is exactly the register layout of
 // v_mfma_f32_32x32x16: a lane supplies 8 consecutive k of one row.
 //
-//   * workgroup tile 256 x 256, K slabs of 64, 8 waves as 4 (M) x 2 (N); a wave
-//     owns 64 x 128 of C (2 x 4 MFMA tiles, 128 accumulator registers) and reads
-//     6 fragments from LDS per 8 MFMAs;
-//   * LDS rows are 144 bytes (64 elements + 8): 16-lane b128 fragment reads hit
-//     16 distinct bank groups;
-//   * two LDS stages: slab s+1 is written while slab s is computed on, one
-//     barrier per slab; global loads (buffer loads, scalar slab offset) run
-//     two slabs ahead in registers; with 16-bit activations and whole slabs the
-//     loads go from global memory straight into a swizzled LDS layout instead;
-//   * fp32 activations are rounded to the weight's 16-bit type on the way
-//     into LDS (round to nearest even), so no conversion pass is needed;
+// Three builds share the tile walk, the operand layout and the epilogue:
+//   * f32 activations, or k not a multiple of 64: workgroup tile 256 x 256, K slabs of
+//     64, 8 waves as 4 (M) x 2 (N), a wave owns 64 x 128 of C; global loads (buffer
+//     loads, scalar slab offset) run two slabs ahead in registers and are rounded to the
+//     weight's 16-bit type on the way into padded LDS rows (144 bytes: 16-lane b128
+//     fragment reads hit 16 distinct bank groups), so no conversion pass is needed;
+//   * 16-bit activations, whole slabs, enough 256-tiles to fill the chip (the default for
+//     the projections): 4 waves, one per SIMD, each owning 128 x 128 of C, slabs fetched
+//     from global memory straight into swizzled, unpadded LDS rows (gemm_ring_kernel);
+//     the same tile with 8 waves is kept behind a knob;
+//   * the same with too few 256-tiles: 128 x 128 tiles, 4 waves, two workgroups per CU;
+//   * two or three products of one A with equal shapes (q/k/v, gate/up) run as one launch
+//     whose tiles cover all of them;
 //   * fixed summation order, no split-K, no atomics: bit-identical run to run.
 #include "attn_device.hpp"
 #include "gemm_kernel.h"
