@@ -35,6 +35,17 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
     // Every load of the lane is issued before the first is used, with clamped addresses
     // instead of predicates: no branch, so nothing waits for an earlier load to come back
     // before the next is sent.
+    // Order of the loads: the token's position (Z-Image) first, because the address of its
+    // rope coefficients depends on it and loads come back in the order they were sent; then
+    // the norm weights, the rows, the rope coefficients. Nothing is used before all are sent.
+    const QkRow qr = qk_row(p.qk, MODE, nullptr, nullptr, seg, tok, true);
+    // weights of this lane's 8 dims: two 16-byte loads whatever the type (no branch between
+    // loads); for 16-bit weights the second repeats the first
+    const void* wsel = (p.w_txt != nullptr && tok < p.qk.txt_rows) ? p.w_txt : p.w;
+    const bool w_f32 = p.w_dtype == kF32;
+    const char* wsrc = static_cast<const char*>(wsel) + d0 * (w_f32 ? 4 : 2);
+    const u32x4 wr0 = *reinterpret_cast<const u32x4*>(wsrc);
+    const u32x4 wr1 = *reinterpret_cast<const u32x4*>(wsrc + (w_f32 ? 16 : 0));
     const TIn* src = reinterpret_cast<const TIn*>(p.x) + (int64_t)seg * p.x_bs + (int64_t)tok * p.x_ts + d0;
     Raw8<TIn> raw[G];
 #pragma unroll
@@ -42,29 +53,29 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
         const int head = h0 + 4 * g;
         raw[g] = ld_raw8<TIn>(src + (int64_t)(head < p.heads ? head : p.heads - 1) * p.x_hs, true);
     }
-    const QkRow qr = qk_row(p.qk, MODE, nullptr, nullptr, seg, tok, true);
     const Rope8 t = ld_rope8(p.qk, MODE, qr, d0);
+    // One wait for everything: the stores below sit under a predicate, and past a branch the
+    // compiler no longer knows how many stores are younger than a load it waits for, so it
+    // would wait for the previous heads' stores as well.
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
     // the token's weights and rope row stay in registers across its heads
-    const void* wsel = (p.w_txt != nullptr && tok < p.qk.txt_rows) ? p.w_txt : p.w;
     f32x4 w0, w1;
-    if (p.w_dtype == kF32) {
-        const float* wf = static_cast<const float*>(wsel) + d0;
-        w0 = *reinterpret_cast<const f32x4*>(wf);
-        w1 = *reinterpret_cast<const f32x4*>(wf + 4);
+    if (w_f32) {
+        w0 = __builtin_bit_cast(f32x4, wr0);
+        w1 = __builtin_bit_cast(f32x4, wr1);
     } else {
-        const u32x4 r = *reinterpret_cast<const u32x4*>(static_cast<const unsigned short*>(wsel) + d0);
         float wv[8];
         if (p.w_dtype == kBF16) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                wv[2 * i] = __builtin_bit_cast(float, r[i] << 16);
-                wv[2 * i + 1] = __builtin_bit_cast(float, r[i] & 0xffff0000u);
+                wv[2 * i] = __builtin_bit_cast(float, wr0[i] << 16);
+                wv[2 * i + 1] = __builtin_bit_cast(float, wr0[i] & 0xffff0000u);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                wv[2 * i] = (float)__builtin_bit_cast(_Float16, (unsigned short)(r[i] & 0xffffu));
-                wv[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(r[i] >> 16));
+                wv[2 * i] = (float)__builtin_bit_cast(_Float16, (unsigned short)(wr0[i] & 0xffffu));
+                wv[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(wr0[i] >> 16));
             }
         }
         w0 = f32x4{wv[0], wv[1], wv[2], wv[3]};
