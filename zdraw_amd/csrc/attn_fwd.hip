@@ -890,8 +890,14 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     }
 }
 
+constexpr int kMaxSplits = 16; // parts per key-split tile
+
 // Combines the parts of the key-split tiles: out[row] = sum_z O_z 2^(m_z - M) / sum_z l_z 2^(m_z - M),
-// M = max_z m_z, z ascending (m_z = -inf: an empty part, weight 0). 32 lanes per row, 4 dims each.
+// M = max_z m_z, z ascending (l_z = 0: an empty part, weight 0). 32 lanes per row, 4 dims each.
+// NZ >= splits is the build's bound on the parts: every load of the lane (reference point and
+// denominator, then the rows, of all parts) is sent before the first is used, so the kernel
+// pays one memory round trip instead of one per part.
+template <int NZ>
 __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnArgs a, int block_rows) {
     const int r = (int)blockIdx.x * 8 + (int)(threadIdx.x >> 5); // row among tail_tiles x block_rows
     const int t = r / block_rows;
@@ -904,32 +910,30 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnArgs a, int b
     const int qrow = qb * block_rows + rr;
     if (qrow >= a.tokens) return;
     const int d0 = (threadIdx.x & 31) * 4;
-    float M = -INFINITY;
-    for (int z = 0; z < a.splits; z++) {
-        const float* ml = a.part_ml + (((int64_t)t * a.splits + z) * block_rows + rr) * 2;
-        M = (ml[1] > 0.f) ? fmaxf(M, ml[0]) : M;
+    const int64_t prow0 = (int64_t)t * a.splits * block_rows + rr;
+    f32x2 ml[NZ];
+    f32x4 x[NZ];
+#pragma unroll
+    for (int z = 0; z < NZ; z++) {
+        ml[z] = f32x2{0.f, 0.f};
+        if (z < a.splits) ml[z] = *reinterpret_cast<const f32x2*>(a.part_ml + (prow0 + (int64_t)z * block_rows) * 2);
     }
+#pragma unroll
+    for (int z = 0; z < NZ; z++) {
+        x[z] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (z < a.splits) x[z] = *reinterpret_cast<const f32x4*>(a.part_o + (prow0 + (int64_t)z * block_rows) * D + d0);
+    }
+    float M = -INFINITY;
+#pragma unroll
+    for (int z = 0; z < NZ; z++) M = (ml[z][1] > 0.f) ? fmaxf(M, ml[z][0]) : M;
     f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
     float l = 0.f;
-    // four parts' loads in flight at a time; parts are still added in ascending order
-    for (int z0 = 0; z0 < a.splits; z0 += 4) {
-        f32x4 x[4];
-        float mz[4], lz[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int z = min(z0 + i, a.splits - 1);
-            const int64_t prow = ((int64_t)t * a.splits + z) * block_rows + rr;
-            mz[i] = a.part_ml[prow * 2];
-            lz[i] = z0 + i < a.splits ? a.part_ml[prow * 2 + 1] : 0.f;
-            x[i] = *reinterpret_cast<const f32x4*>(a.part_o + prow * D + d0);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            if (!(lz[i] > 0.f)) continue; // past the last part, or a part that admitted no key
-            const float w = __builtin_amdgcn_exp2f(mz[i] - M);
-            l += lz[i] * w;
-            acc += x[i] * w;
-        }
+    for (int z = 0; z < NZ; z++) {
+        // past the last part, or a part that admitted no key: weight 0 (its row is all zeros)
+        const float w = (ml[z][1] > 0.f) ? __builtin_amdgcn_exp2f(ml[z][0] - M) : 0.f;
+        l += ml[z][1] * w;
+        acc += x[z] * w;
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     acc *= inv;
@@ -969,7 +973,11 @@ static hipError_t launch_one(const AttnArgs& a0, hipStream_t stream) {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         const int rows = tail * NW * 32 * QB;
-        attn_merge_kernel<<<dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream>>>(a, NW * 32 * QB);
+        const dim3 mgrid((unsigned)((rows + 7) / 8));
+        if (a.splits <= 4) attn_merge_kernel<4><<<mgrid, dim3(256), 0, stream>>>(a, NW * 32 * QB);
+        else if (a.splits <= 8) attn_merge_kernel<8><<<mgrid, dim3(256), 0, stream>>>(a, NW * 32 * QB);
+        else if (a.splits <= kMaxSplits) attn_merge_kernel<kMaxSplits><<<mgrid, dim3(256), 0, stream>>>(a, NW * 32 * QB);
+        else return hipErrorInvalidValue;
         return hipGetLastError();
     }
     return hipSuccess;
@@ -1039,7 +1047,7 @@ void attention_tail_plan(int64_t tiles, int cus, int key_blocks, int* tail_tiles
     // fills them all; each part keeps at least 8 key blocks
     if (tail == 0 || tail * 2 > cus) return;
     int s = cus / tail;
-    if (s > 16) s = 16;
+    if (s > fwd::kMaxSplits) s = fwd::kMaxSplits;
     if (s > key_blocks / 8) s = key_blocks / 8;
     if (s < 2) return;
     *tail_tiles = tail;
