@@ -572,9 +572,9 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
     store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, l32, h);
 }
 
-// Measured on the Klein projections, same box: eight waves (two per SIMD, 64 x 128 each)
-// 1048-1217 TFLOP/s; four waves with the schedule above 1047-1248; four waves with the simple
-// loop of the eight-wave build 960-1120.
+// Measured on the Klein projections, same box, all with row-by-row stores and row-major tile
+// order: eight waves (two per SIMD, 64 x 128 each) 1048-1217 TFLOP/s; four waves with the
+// schedule above 1047-1248; four waves with the simple loop of the eight-wave build 960-1120.
 constexpr int DMA_WM = 4, DMA_WN = 2;
 
 static int g_gemm_build = 1; // 256-tiles of 16-bit activations: 1 = four-wave build (default), 0 = eight-wave build (measurement knob)
