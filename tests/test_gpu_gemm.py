@@ -350,3 +350,31 @@ def test_many_tile_problem_runs_the_256_tile_builds(ctx, build, c_dtype):
         tol = 2 ** -8 * np.abs(want).max() + 1e-4
     # rows and columns of the ragged edge tiles
     assert np.abs(got[-1] - want[-1]).max() < tol and np.abs(got[:, -1] - want[:, -1]).max() < tol
+
+
+@pytest.mark.parametrize("wdt", [hip.W_BF16, hip.W_F16])
+@pytest.mark.parametrize("ldc", [256, 251])
+def test_small_tile_build_16_bit_output_edges_and_pitch(ctx, wdt, ldc):
+    # Few tiles, 16-bit activations, k a multiple of 64: the 128-tile build. With rows of C on
+    # 16 bytes (ldc 256) its 16-bit output leaves through LDS as whole rows: the last rows
+    # (m = 200 of 256) must not be stored, the last column chunk (n = 250: two of eight
+    # columns) goes element by element, and the pad columns of the pitch stay untouched. With
+    # ldc 251 the rows are not aligned and the direct stores run instead. Same results.
+    rng = np.random.default_rng(5 + ldc)
+    m, k, n = 200, 128, 250
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
+    a_bits, ar = to16(a, wdt)
+    w_bits, wr = to16(w, wdt)
+    adt = act_dtype(wdt)
+    guard = 64  # elements behind the last row: must stay as they were
+    init = np.full(m * ldc + guard, 0x7e7e, np.uint16)
+    raw = run_ext(ctx, a_bits, w_bits, m, k, n, wdt, adt, adt, ldc=ldc, c_init=init.view(np.uint8))
+    flat = raw.view(np.uint16)
+    assert (flat[m * ldc:] == 0x7e7e).all()
+    full = flat[:m * ldc].reshape(m, ldc)
+    assert (full[:, n:] == 0x7e7e).all()
+    got = from16(full[:, :n], wdt)
+    want = from16(to16(zo.linear_batch(ar, wr), wdt)[0], wdt)
+    ulp = 2.0 ** -7 if wdt == hip.W_BF16 else 2.0 ** -10
+    assert np.abs(got - want).max() <= ulp * np.abs(want).max() + 1e-5

@@ -118,52 +118,57 @@ __device__ __forceinline__ void store_tile(const GemmArgs& g, void* c, const f32
     }
 }
 
-// The same block of C (4 x 4 tiles of one wave of the four-wave build) for a 16-bit C, by way
-// of LDS: stored straight from the accumulation layout a lane's 8 bytes make every store
-// instruction 32 separate 16-byte pieces; turned through a wave-private 128 x 272-byte region
-// of the (by then idle) slab ring, every instruction stores four whole 256-byte rows.
+// The same block of C for a 16-bit C, by way of LDS: stored straight from the accumulation
+// layout a lane's 8 bytes make every store instruction 32 separate 16-byte pieces; turned
+// through a wave-private region of the (by then idle) slab stages, (32 TM) rows of
+// epi_pitch(TN) bytes, every instruction stores whole rows of the block (four 256-byte rows
+// for TN = 4, eight 128-byte rows for TN = 2).
 // Needs: every direct load of the workgroup has landed and a barrier has passed since the last
 // fragment read; 16-byte aligned rows of C.
-constexpr int EPI_PITCH = 272; // bytes per staged row: 256 + 16, keeps 16-byte alignment and spreads the banks
-constexpr size_t kRingLdsBytes = 4 * (size_t)128 * EPI_PITCH; // >= the two 64 KB slab stages
-template <bool F16, typename TC>
-__device__ __forceinline__ void store_tile_lds(const GemmArgs& g, void* c, const f32x16 (&acc)[4][4], unsigned lds_wave, int row0, int col0, int lane) {
+constexpr int epi_pitch(int tn) { return 64 * tn + 16; } // bytes per staged row: keeps 16-byte alignment, spreads the banks
+constexpr size_t kRingLdsBytes = 4 * (size_t)128 * epi_pitch(4); // four-wave build: >= its two 64 KB slab stages
+template <bool F16, typename TC, int TM, int TN>
+__device__ __forceinline__ void store_tile_lds(const GemmArgs& g, void* c, const f32x16 (&acc)[TM][TN], unsigned lds_wave, int row0, int col0, int lane) {
     static_assert(sizeof(TC) == 2, "16-bit C only");
+    constexpr int PITCH = epi_pitch(TN);
+    constexpr int CH = 4 * TN;   // 16-byte chunks per staged row
+    constexpr int RPI = 64 / CH; // rows per read-back instruction
+    constexpr int NQ = 32 * TM / RPI;
     typedef __attribute__((address_space(3))) u32x2* lds_u32x2_t;
     typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
     const int l32 = lane & 31, h = lane >> 5;
-    const unsigned wbase = lds_wave + (unsigned)(l32 * EPI_PITCH + h * 8);
+    const unsigned wbase = lds_wave + (unsigned)(l32 * PITCH + h * 8);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < TM; i++) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < TN; j++) {
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const f32x4 v = f32x4{acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2], acc[i][j][4 * r + 3]};
                 u32x2 pk;
                 if constexpr (F16) pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4));
                 else pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
-                *(lds_u32x2_t)(wbase + (unsigned)(i * 32 * EPI_PITCH + j * 64 + r * 16)) = pk;
+                *(lds_u32x2_t)(wbase + (unsigned)(i * 32 * PITCH + j * 64 + r * 16)) = pk;
             }
         }
         __builtin_amdgcn_sched_barrier(0);
     }
-    // lane -> row 4 q + lane / 16, columns 8 (lane % 16) .. + 8
-    const int rr = lane >> 4, ch = lane & 15;
+    // lane -> row RPI q + lane / CH, columns 8 (lane % CH) .. + 8
+    const int rr = lane / CH, ch = lane % CH;
     const int col = col0 + 8 * ch;
-    const unsigned rbase = lds_wave + (unsigned)(rr * EPI_PITCH + ch * 16);
+    const unsigned rbase = lds_wave + (unsigned)(rr * PITCH + ch * 16);
     unsigned short* const cbase = reinterpret_cast<unsigned short*>(c) + (int64_t)(row0 + rr) * g.ldc + col;
     const bool whole = col + 8 <= g.n;
 #pragma unroll
-    for (int q0 = 0; q0 < 32; q0 += 8) {
+    for (int q0 = 0; q0 < NQ; q0 += 8) {
         u32x4 v[8];
 #pragma unroll
-        for (int q = 0; q < 8; q++) v[q] = *(lds_u32x4_t)(rbase + (unsigned)((q0 + q) * 4 * EPI_PITCH));
+        for (int q = 0; q < 8; q++) v[q] = *(lds_u32x4_t)(rbase + (unsigned)((q0 + q) * RPI * PITCH));
 #pragma unroll
         for (int q = 0; q < 8; q++) {
-            const int row = row0 + 4 * (q0 + q) + rr;
+            const int row = row0 + RPI * (q0 + q) + rr;
             if (row >= g.m) continue;
-            unsigned short* const dst = cbase + (int64_t)(4 * (q0 + q)) * g.ldc;
+            unsigned short* const dst = cbase + (int64_t)(RPI * (q0 + q)) * g.ldc;
             if (whole) {
                 *reinterpret_cast<u32x4*>(dst) = v[q];
             } else {
@@ -434,6 +439,15 @@ __global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArg
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): slab s+1 has landed
         __syncthreads();
     }
+    if constexpr (sizeof(TC) == 2 && TB == 128) {
+        // the loop's last barrier has left the stages idle; the staged tile fits into them
+        static_assert((size_t)WM * WN * 32 * TM * epi_pitch(TN) <= 2 * (size_t)(2 * TB * BK * 2), "staging exceeds the slab stages");
+        if ((g.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(cp) % 16 == 0)) {
+            store_tile_lds<F16, TC, TM, TN>(g, cp, acc, lds_address(smem) + (unsigned)wave * (32 * TM * epi_pitch(TN)),
+                                            m0 + wm * (32 * TM), n0 + wn * (32 * TN), lane);
+            return;
+        }
+    }
     store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * (32 * TM), n0 + wn * (32 * TN), l32, h);
 }
 
@@ -565,7 +579,7 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         // uniform over the launch: rows of C start on 16 bytes
         if ((g.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(cp) % 16 == 0)) {
             __syncthreads(); // every wave's loads have landed and its fragments are read: the ring is idle
-            store_tile_lds<F16, TC>(g, cp, acc, lds0 + (unsigned)wave * (128 * EPI_PITCH), m0 + wm * 128, n0 + wn * 128, lane);
+            store_tile_lds<F16, TC, TM, TN>(g, cp, acc, lds0 + (unsigned)wave * (128 * epi_pitch(TN)), m0 + wm * 128, n0 + wn * 128, lane);
             return;
         }
     }
