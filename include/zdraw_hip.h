@@ -234,6 +234,14 @@ int zdraw_hip_run_gemm_triple(void* queue, void* pipeline, void* a, void* w0, vo
  * from the concat operand at its row pitch. */
 int zdraw_hip_run_gemm_ext_enc(void* batch, void* a, void* w, void* c, const ZdrawGemmParams* params,
                                const ZdrawHipGemmExt* ext);
+/* The general form for `count` (1..3) products of one A that share `ext` (gate/up, q/k/v of
+ * the resident 16-bit path; the pair/triple of metal_c.zig:175-198 with the options of the
+ * entry above): equal shapes and weight types run as one launch whose tiles cover all of
+ * them, otherwise one launch each. params[i]->weight_offset selects each W; ext->c_off
+ * applies to every C. A product this backend does not run refuses the whole call (1)
+ * before anything is enqueued. */
+int zdraw_hip_run_gemm_group_ext_enc(void* batch, void* a, void* const* ws, void* const* cs,
+                                     const ZdrawGemmParams* const* params, uint32_t count, const ZdrawHipGemmExt* ext);
 
 /* ---- Z-Image layer, attention segment --------------------------------------
  * The q/k/v projections, QK-norm + rope, attention and output projection of one
@@ -294,7 +302,8 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
 
 /* ---- library-owned scratch (metal_c.zig:321-325) -------------------------- */
 /* Grow-only, process-lifetime, filled at (re)allocation with 0x00 (0xFF when
- * ZDRAW_SCRATCH_POISON is set, metal_api.m:6147-6181). slot in [0, 5). */
+ * ZDRAW_SCRATCH_POISON is set, metal_api.m:6147-6181). slot in [0, 6): 0-2 prepared
+ * operands, 3-4 the parts of key-split attention tiles, 5 the parts of k-split GEMM tiles. */
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes);
 
 /* ---- counters and timing (metal_api.m:333-353, 420-433) ------------------- */
@@ -349,6 +358,14 @@ void zdraw_hip_set_attention_variant(int variant);
  * at most 16 parts; *tail_tiles = 0 and *splits = 1 when everything runs whole. */
 void zdraw_hip_attention_tail_plan(uint64_t tiles, uint32_t cus, uint32_t key_blocks, uint32_t* tail_tiles,
                                    uint32_t* splits);
+
+/* The same for `groups` (1..3) side-by-side products C[m][n] = A[m][k] x W[n][k]^T of 16-bit
+ * activations: the tiles are 256 x 256; a last round that fills at most half the CUs runs as
+ * *splits ranges of k per tile (at most 8, at least four 64-wide slabs each) whose fp32
+ * partial tiles are added in range order; nothing is split when k is not a multiple of 64,
+ * when fewer than 160 tiles exist, or under the eight-wave build. */
+void zdraw_hip_gemm_tail_plan(uint32_t m, uint32_t k, uint32_t n, uint32_t groups, uint32_t cus, uint32_t* tail_tiles,
+                              uint32_t* splits);
 
 /* Measurement knob: which build multiplies 256 x 256 tiles of 16-bit activations.
  * 1 = four waves, 128 x 128 each (default); 0 = eight waves, 64 x 128 each. */

@@ -59,6 +59,30 @@ def test_abi_struct_sizes():
     assert "#define ZDRAW_HIP_ABI_GEMM_EXT_SIZE 48" in text
 
 
+def test_gemm_tail_plan_of_the_projection_shapes():
+    # 256 CUs, 256 x 256 tiles of C: which last rounds of the projections are split along k
+    L = hip.lib()
+
+    def plan(m, k, n, groups=1, cus=256):
+        t, s = C.c_uint32(99), C.c_uint32(99)
+        L.zdraw_hip_gemm_tail_plan(m, k, n, groups, cus, C.byref(t), C.byref(s))
+        return t.value, s.value
+
+    assert plan(4608, 3072, 9216) == (0, 1)          # Klein q/k/v: 648 tiles, a tail of 136 stays whole
+    assert plan(4608, 3840, 3840, 3) == (42, 6)      # Z-Image q/k/v group: 810 tiles = 3 rounds + 42
+    assert plan(4608, 3840, 3840) == (14, 8)         # Z-Image out projection: 270 tiles, never more than 8 parts
+    assert plan(4608, 12288, 3072) == (0, 1)         # 216 tiles: one partly filled round, nothing before it to balance
+    assert plan(512, 3072, 9216) == (0, 1)           # fewer than 160 tiles: the 128-tile build
+    assert plan(4322, 1216, 4090) == (16, 4)         # 272 tiles, 19 slabs: at least four slabs per part
+    assert plan(4322, 128, 4090) == (0, 1)           # two slabs: too short to split
+    assert plan(4322, 1220, 4090) == (0, 1)          # k not a multiple of 64: another build
+    assert plan(4608, 3840, 3840, 3, cus=0) == (0, 1) and plan(0, 64, 64) == (0, 1)
+    for mt in range(10, 40):                         # invariants
+        t, s = plan(mt * 256, 2048, 16 * 256)
+        tiles = mt * 16
+        assert (t == 0 and s == 1) or (tiles >= 160 and t == tiles % 256 and 2 <= s <= 8 and t * s <= 256 and 32 // s >= 4)
+
+
 def test_tail_plan_of_the_baseline_shapes():
     # 256 CUs, one 256-row tile per workgroup: which last rounds are split along the keys
     L = hip.lib()

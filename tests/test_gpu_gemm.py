@@ -378,3 +378,104 @@ def test_small_tile_build_16_bit_output_edges_and_pitch(ctx, wdt, ldc):
     want = from16(to16(zo.linear_batch(ar, wr), wdt)[0], wdt)
     ulp = 2.0 ** -7 if wdt == hip.W_BF16 else 2.0 ** -10
     assert np.abs(got - want).max() <= ulp * np.abs(want).max() + 1e-5
+
+
+def _split_tail_case(rng, m, k, n):
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
+    a_bits, ar = to16(a, hip.W_BF16)
+    w_bits, wr = to16(w, hip.W_BF16)
+    return a_bits, ar, w_bits, wr
+
+
+@pytest.mark.parametrize("c_dtype", [hip.BF16, hip.F32])
+def test_k_split_last_round_matches_whole_tiles_and_oracle(ctx, c_dtype):
+    # 17 x 16 = 272 tiles of 256 x 256 on 256 CUs: the 16 tiles of the second round run as 4
+    # ranges of k each (19 slabs: 5, 5, 5, 4) and are put together by the merge kernel; ragged
+    # last row and column of tiles, pitch wider than the row. Checked against the oracle on
+    # identically rounded operands (rows of the split tiles and rows elsewhere), against an
+    # fp32 product of the whole matrix, against the eight-wave build (which never splits), and
+    # for bit-equal reruns.
+    L = hip.lib()
+    m, k, n, ldc = 4322, 1216, 4090, 4096
+    t, s = C.c_uint32(), C.c_uint32()
+    L.zdraw_hip_gemm_tail_plan(m, k, n, 1, 256, C.byref(t), C.byref(s))
+    assert (t.value, s.value) == (16, 4)
+    a_bits, ar, w_bits, wr = _split_tail_case(np.random.default_rng(41), m, k, n)
+    esz = 4 if c_dtype == hip.F32 else 2
+    init = np.full(m * ldc * esz, 0x5a, np.uint8)
+
+    def run(build):
+        L.zdraw_hip_set_gemm_build(build)
+        try:
+            raw = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, c_dtype, ldc=ldc, c_init=init)
+        finally:
+            L.zdraw_hip_set_gemm_build(1)
+        if c_dtype == hip.F32:
+            full = raw.view(np.float32).reshape(m, ldc)
+            assert (raw.reshape(m, ldc * 4)[:, n * 4:] == 0x5a).all()
+            return full[:, :n].copy()
+        full = raw.view(np.uint16).reshape(m, ldc)
+        assert (full[:, n:] == 0x5a5a).all()  # the pad columns of the pitch stay untouched
+        return from16(full[:, :n], hip.W_BF16)
+
+    got = run(1)
+    assert np.array_equal(got, run(1))
+    whole = run(0)
+    scale = np.sqrt(k) * np.sqrt(np.mean(ar.astype(np.float64) ** 2)) * np.sqrt(np.mean(wr.astype(np.float64) ** 2))
+    ulp = 2.0 ** -8 * max(np.abs(whole).max(), 1.0) if c_dtype == hip.BF16 else 0.0
+    assert np.abs(got - whole).max() <= 2 * ulp + 2e-5 * scale  # same products, another summation order
+    ref32 = ar @ wr.T
+    assert np.abs(got - ref32).max() <= ulp + 1e-4 * scale
+    rows = np.unique(np.concatenate([np.arange(m - 300, m), np.random.default_rng(3).choice(m - 300, 200, replace=False)]))
+    want = zo.linear_batch(ar[rows], wr)
+    assert np.abs(got[rows] - want).max() <= ulp + 2e-5 * scale
+
+
+def test_k_split_last_round_of_a_group(ctx):
+    # two products of one bf16 A through the grouped entry: 2 x (17 x 8) = 272 tiles, the 16
+    # split tiles all belong to the second product; against the oracle and the one-by-one runs
+    L = hip.lib()
+    m, k, n = 4322, 1216, 2040
+    t, s = C.c_uint32(), C.c_uint32()
+    L.zdraw_hip_gemm_tail_plan(m, k, n, 2, 256, C.byref(t), C.byref(s))
+    assert (t.value, s.value) == (16, 4)
+    rng = np.random.default_rng(43)
+    a_bits, ar, w0_bits, w0r = _split_tail_case(rng, m, k, n)
+    w1 = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
+    w1_bits, w1r = to16(w1, hip.W_BF16)
+    ab = ctx.buffer(a_bits)
+    wb = ctx.buffer(np.concatenate([w0_bits.ravel(), w1_bits.ravel()]))
+    cbs = [ctx.buffer(np.zeros(m * n, np.uint16)) for _ in range(2)]
+    ps = [hip.GemmParams(m, k, n, hip.W_BF16, hip.GEMM_HALF, off) for off in (0, n * k * 2)]
+    ext = hip.GemmExt(0, 0, 0, 0, 0, hip.BF16, hip.BF16)
+    ws = (C.c_void_p * 2)(wb.handle, wb.handle)
+    cs = (C.c_void_p * 2)(cbs[0].handle, cbs[1].handle)
+    pp = (C.POINTER(hip.GemmParams) * 2)(C.pointer(ps[0]), C.pointer(ps[1]))
+    d0 = L.zdraw_hip_dispatch_count()
+    batch = L.zdraw_hip_batch_begin(ctx.queue)
+    rc = L.zdraw_hip_run_gemm_group_ext_enc(batch, ab.handle, ws, cs, pp, 2, C.byref(ext))
+    assert L.zdraw_hip_batch_end(batch) == 0
+    assert rc == 0, hip.last_error()
+    assert L.zdraw_hip_dispatch_count() - d0 == 1
+    scale = np.sqrt(k) * np.sqrt(np.mean(ar.astype(np.float64) ** 2)) * np.sqrt(np.mean(w0r.astype(np.float64) ** 2))
+    rows = np.unique(np.concatenate([np.arange(m - 300, m), np.arange(0, m - 300, 37)]))
+    for i, wr in enumerate((w0r, w1r)):
+        got = from16(cbs[i].read(np.uint16, (m, n)), hip.W_BF16)
+        ulp = 2.0 ** -8 * max(np.abs(got).max(), 1.0)
+        assert np.abs(got - ar @ wr.T).max() <= ulp + 1e-4 * scale
+        assert np.abs(got[rows] - zo.linear_batch(ar[rows], wr)).max() <= ulp + 2e-5 * scale
+        one = run_ext(ctx, a_bits, np.concatenate([w0_bits.ravel(), w1_bits.ravel()]), m, k, n, hip.W_BF16, hip.BF16, hip.BF16)
+        if i == 0:
+            assert np.abs(from16(one.view(np.uint16).reshape(m, n), hip.W_BF16) - got).max() <= 2 * ulp + 2e-5 * scale
+    # a count outside 1..3 and a product this backend does not run leave nothing enqueued
+    d0 = L.zdraw_hip_dispatch_count()
+    batch = L.zdraw_hip_batch_begin(ctx.queue)
+    assert L.zdraw_hip_run_gemm_group_ext_enc(batch, ab.handle, ws, cs, pp, 4, C.byref(ext)) < 0
+    bad = hip.GemmParams(m, k, n, hip.W_F32, hip.GEMM_HALF, 0)
+    pp_bad = (C.POINTER(hip.GemmParams) * 2)(C.pointer(ps[0]), C.pointer(bad))
+    assert L.zdraw_hip_run_gemm_group_ext_enc(batch, ab.handle, ws, cs, pp_bad, 2, C.byref(ext)) == 1
+    assert L.zdraw_hip_batch_end(batch) == 0
+    assert L.zdraw_hip_dispatch_count() == d0
+    for b in [ab, wb] + cbs:
+        b.release()

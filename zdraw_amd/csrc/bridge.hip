@@ -551,7 +551,7 @@ int finish_blocking(Queue* qu, hipEvent_t start, hipEvent_t stop) {
     return ZDRAW_HIP_OK;
 }
 
-Buffer* g_scratch[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+Buffer* g_scratch[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 
 bool scratch_poisoned(int slot) {
     // ZDRAW_SCRATCH_POISON: "1" every slot, "attn" the group, "attn:2" one slot
@@ -568,8 +568,8 @@ bool scratch_poisoned(int slot) {
 // One launch for `groups` (1..3) products that share A, every dimension and the
 // extension block: group i multiplies by ws[i] at byte offset w_offs[i] into cs[i].
 int enqueue_gemm_group(void* a, void* const* ws, void* const* cs, const uint64_t* w_offs, int groups,
-                       const ZdrawGemmParams* p, const ZdrawHipGemmExt* x, hipStream_t stream) {
-    if (!p || !x || groups < 1 || groups > 3) {
+                       const ZdrawGemmParams* p, const ZdrawHipGemmExt* x, Queue* queue) {
+    if (!p || !x || !queue || groups < 1 || groups > 3) {
         set_err("null params");
         return ZDRAW_HIP_ERR_HANDLE;
     }
@@ -625,7 +625,23 @@ int enqueue_gemm_group(void* a, void* const* ws, void* const* cs, const uint64_t
     g.tiles_n = (int32_t)((p->n + (uint32_t)gemm_tile_cols() - 1) / (uint32_t)gemm_tile_cols());
     if ((uint64_t)g.tiles_n * (uint64_t)groups * ((p->m + (uint32_t)gemm_tile_rows() - 1) / (uint32_t)gemm_tile_rows()) > 0x7fffffffull)
         return unavailable("grid too large");
-    hipError_t e = launch_gemm(g, (int)x->a_dtype, (int)wt, (int)x->c_dtype, stream);
+    {
+        // a last round of tiles that fills at most half the CUs runs split along k; its fp32
+        // partial tiles go through scratch slot 5
+        int tail = 0, splits = 1;
+        gemm_tail_plan(g, (int)x->a_dtype, queue->dev->cus, &tail, &splits);
+        if (splits > 1) {
+            Buffer* part = static_cast<Buffer*>(zdraw_hip_attn_scratch(queue->dev, 5, gemm_part_bytes(tail, splits)));
+            if (!part) {
+                set_err("scratch allocation failed");
+                return ZDRAW_HIP_ERR_HANDLE;
+            }
+            g.splits = splits;
+            g.tile_base = tail; // launch_gemm reads the tail size here
+            g.part = static_cast<float*>(part->ptr);
+        }
+    }
+    hipError_t e = launch_gemm(g, (int)x->a_dtype, (int)wt, (int)x->c_dtype, queue->stream);
     if (e != hipSuccess) {
         set_err("gemm launch: %s", hipGetErrorString(e));
         return ZDRAW_HIP_ERR_HANDLE;
@@ -634,12 +650,12 @@ int enqueue_gemm_group(void* a, void* const* ws, void* const* cs, const uint64_t
     return ZDRAW_HIP_OK;
 }
 
-int enqueue_gemm(void* a, void* w, void* c, const ZdrawGemmParams* p, const ZdrawHipGemmExt* x, hipStream_t stream) {
+int enqueue_gemm(void* a, void* w, void* c, const ZdrawGemmParams* p, const ZdrawHipGemmExt* x, Queue* queue) {
     if (!p) {
         set_err("null params");
         return ZDRAW_HIP_ERR_HANDLE;
     }
-    return enqueue_gemm_group(a, &w, &c, &p->weight_offset, 1, p, x, stream);
+    return enqueue_gemm_group(a, &w, &c, &p->weight_offset, 1, p, x, queue);
 }
 
 } // namespace
@@ -942,7 +958,7 @@ int zdraw_hip_run_gemm_ext_enc(void* batch, void* a, void* w, void* c, const Zdr
         set_err("null batch");
         return ZDRAW_HIP_ERR_HANDLE;
     }
-    return enqueue_gemm(a, w, c, params, ext, b->queue->stream);
+    return enqueue_gemm(a, w, c, params, ext, b->queue);
 }
 
 int zdraw_hip_run_gemm_off_enc(void* batch, void* pipeline, void* a, void* w, void* c,
@@ -991,6 +1007,31 @@ int zdraw_hip_run_gemm(void* queue, void* pipeline, void* a, void* w, void* c, c
 namespace {
 // Two or three products of the same f32 A (metal_api.m zdraw_metal_run_gemm_pair / _triple):
 // one grouped launch when the shapes and weight types agree, one launch each otherwise.
+// `count` products of one A into an open batch: one grouped launch when shapes and weight
+// types agree, else one launch each; a product this backend does not run refuses the call
+// before anything is enqueued.
+int enqueue_gemm_several(Batch* b, void* a, void* const* ws, void* const* cs, const ZdrawGemmParams* const* ps, int count,
+                         const ZdrawHipGemmExt* x) {
+    for (int i = 0; i < count; i++) {
+        if (ps[i]->mode != ZDRAW_HIP_GEMM_HALF || (ps[i]->dtype != ZDRAW_HIP_W_F16 && ps[i]->dtype != ZDRAW_HIP_W_BF16) ||
+            (ps[i]->k % 8 != 0 && ps[i]->m != 0 && ps[i]->k != 0 && ps[i]->n != 0))
+            return unavailable("a product of the group is not a 16-bit-weight half-mode GEMM with k % 8 == 0");
+    }
+    bool same = true;
+    for (int i = 1; i < count; i++)
+        same = same && ps[i]->m == ps[0]->m && ps[i]->k == ps[0]->k && ps[i]->n == ps[0]->n &&
+               ps[i]->dtype == ps[0]->dtype && ps[i]->mode == ps[0]->mode;
+    int rc = ZDRAW_HIP_OK;
+    if (same) {
+        uint64_t offs[3];
+        for (int i = 0; i < count; i++) offs[i] = ps[i]->weight_offset;
+        rc = enqueue_gemm_group(a, ws, cs, offs, count, ps[0], x, b->queue);
+    } else {
+        for (int i = 0; i < count && rc == ZDRAW_HIP_OK; i++) rc = enqueue_gemm(a, ws[i], cs[i], ps[i], x, b->queue);
+    }
+    return rc;
+}
+
 int run_gemm_several(void* queue, void* pipeline, void* a, void* const* ws, void* const* cs,
                      const ZdrawGemmParams* const* ps, int count) {
     int rc = check_pipeline(pipeline, 0, 2);
@@ -1009,29 +1050,26 @@ int run_gemm_several(void* queue, void* pipeline, void* a, void* const* ws, void
     memset(&x, 0, sizeof(x));
     x.a_dtype = ZDRAW_HIP_F32;
     x.c_dtype = ZDRAW_HIP_F32;
-    // a product this backend does not run refuses the call before anything is enqueued
-    for (int i = 0; i < count; i++) {
-        if (ps[i]->mode != ZDRAW_HIP_GEMM_HALF || (ps[i]->dtype != ZDRAW_HIP_W_F16 && ps[i]->dtype != ZDRAW_HIP_W_BF16) ||
-            (ps[i]->k % 8 != 0 && ps[i]->m != 0 && ps[i]->k != 0 && ps[i]->n != 0)) {
-            zdraw_hip_batch_end(b);
-            return unavailable("a product of the group is not a 16-bit-weight half-mode GEMM with k % 8 == 0");
-        }
-    }
-    bool same = true;
-    for (int i = 1; i < count; i++)
-        same = same && ps[i]->m == ps[0]->m && ps[i]->k == ps[0]->k && ps[i]->n == ps[0]->n &&
-               ps[i]->dtype == ps[0]->dtype && ps[i]->mode == ps[0]->mode;
-    if (same) {
-        uint64_t offs[3];
-        for (int i = 0; i < count; i++) offs[i] = ps[i]->weight_offset;
-        rc = enqueue_gemm_group(a, ws, cs, offs, count, ps[0], &x, b->queue->stream);
-    } else {
-        for (int i = 0; i < count && rc == ZDRAW_HIP_OK; i++) rc = enqueue_gemm(a, ws[i], cs[i], ps[i], &x, b->queue->stream);
-    }
+    rc = enqueue_gemm_several(b, a, ws, cs, ps, count, &x);
     const int rc2 = zdraw_hip_batch_end(b);
     return rc != ZDRAW_HIP_OK ? rc : rc2;
 }
 } // namespace
+
+int zdraw_hip_run_gemm_group_ext_enc(void* batch, void* a, void* const* ws, void* const* cs,
+                                     const ZdrawGemmParams* const* params, uint32_t count, const ZdrawHipGemmExt* ext) {
+    Batch* b = static_cast<Batch*>(batch);
+    if (!b || !ws || !cs || !params || !ext || count < 1 || count > 3) {
+        set_err("null batch, arrays or ext, or count outside 1..3");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    for (uint32_t i = 0; i < count; i++)
+        if (!params[i]) {
+            set_err("null params");
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+    return enqueue_gemm_several(b, a, ws, cs, params, (int)count, ext);
+}
 
 int zdraw_hip_run_gemm_pair(void* queue, void* pipeline, void* a, void* w0, void* c0, const ZdrawGemmParams* params0,
                             void* w1, void* c1, const ZdrawGemmParams* params1) {
@@ -1116,19 +1154,19 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
         void* const wsv[3] = {w->q, w->k, w->v};
         void* const csv[3] = {bufs->q, bufs->k, bufs->v};
         const uint64_t offs[3] = {p->q.weight_offset, p->k.weight_offset, p->v.weight_offset};
-        if ((rc = enqueue_gemm_group(bufs->norm, wsv, csv, offs, 3, &p->q, &gx, st)) != ZDRAW_HIP_OK) return rc;
+        if ((rc = enqueue_gemm_group(bufs->norm, wsv, csv, offs, 3, &p->q, &gx, b->queue)) != ZDRAW_HIP_OK) return rc;
     } else {
-        if ((rc = enqueue_gemm(bufs->norm, w->q, bufs->q, &p->q, &gx, st)) != ZDRAW_HIP_OK) return rc;
-        if ((rc = enqueue_gemm(bufs->norm, w->k, bufs->k, &p->k, &gx, st)) != ZDRAW_HIP_OK) return rc;
-        if ((rc = enqueue_gemm(bufs->norm, w->v, bufs->v, &p->v, &gx, st)) != ZDRAW_HIP_OK) return rc;
+        if ((rc = enqueue_gemm(bufs->norm, w->q, bufs->q, &p->q, &gx, b->queue)) != ZDRAW_HIP_OK) return rc;
+        if ((rc = enqueue_gemm(bufs->norm, w->k, bufs->k, &p->k, &gx, b->queue)) != ZDRAW_HIP_OK) return rc;
+        if ((rc = enqueue_gemm(bufs->norm, w->v, bufs->v, &p->v, &gx, b->queue)) != ZDRAW_HIP_OK) return rc;
     }
     if ((rc = enqueue(plan, st)) != ZDRAW_HIP_OK) return rc;
-    return enqueue_gemm(bufs->mix, w->proj, bufs->attn, &p->proj, &gx, st);
+    return enqueue_gemm(bufs->mix, w->proj, bufs->attn, &p->proj, &gx, b->queue);
 }
 
 // ------------------------------------------------------------------ scratch
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes) {
-    if (!device || slot < 0 || slot >= 5 || bytes == 0) return nullptr;
+    if (!device || slot < 0 || slot >= 6 || bytes == 0) return nullptr;
     Buffer* cur = g_scratch[slot];
     if (cur && cur->len >= bytes) return cur;
     // Grow: work already enqueued may still read the old allocation, so drain
@@ -1237,6 +1275,19 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
 void zdraw_hip_set_attention_variant(int variant) { g_variant = variant & 3; }
 
 void zdraw_hip_set_gemm_build(int build) { gemm_set_build(build); }
+
+void zdraw_hip_gemm_tail_plan(uint32_t m, uint32_t k, uint32_t n, uint32_t groups, uint32_t cus, uint32_t* tail_tiles,
+                              uint32_t* splits) {
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.m = (int32_t)m; g.k = (int32_t)k; g.n = (int32_t)n;
+    g.groups = (int32_t)groups;
+    int t = 0, s = 1;
+    if (m && k && n && groups >= 1 && groups <= 3 && m <= 0x7fffffffu && k <= 0x7fffffffu && n <= 0x7fffffffu)
+        gemm_tail_plan(g, (int)ZDRAW_HIP_BF16, (int)cus, &t, &s);
+    if (tail_tiles) *tail_tiles = (uint32_t)t;
+    if (splits) *splits = (uint32_t)s;
+}
 
 void zdraw_hip_attention_tail_plan(uint64_t tiles, uint32_t cus, uint32_t key_blocks, uint32_t* tail_tiles,
                                    uint32_t* splits) {

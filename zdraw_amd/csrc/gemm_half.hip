@@ -472,7 +472,15 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
     const int l32 = lane & 31;
     const int h = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
-    const int logical = logical_tile();
+    // a tile of the split last round: workgroup = (tile, part), the part is a range of slabs
+    int logical, part_id = 0;
+    if (g.splits > 1) {
+        const int t = (int)blockIdx.x / g.splits;
+        part_id = (int)blockIdx.x - t * g.splits;
+        logical = g.tile_base + t;
+    } else {
+        logical = logical_tile();
+    }
     const int tiles_row = g.tiles_n * g.groups;
     int tm, tn;
     tile_coords(logical, (g.m + BM - 1) / BM, tiles_row, tm, tn);
@@ -498,12 +506,17 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         a_off[j] = ((unsigned)ar * (unsigned)g.lda + (unsigned)(c * 8)) * 2u;
         w_off[j] = ((unsigned)wr * (unsigned)g.ldw + (unsigned)(c * 8)) * 2u;
     }
-    const int nslab = g.k / BK;
+    int nslab = g.k / BK, slab0 = 0;
+    if (g.splits > 1) {
+        const int per = (nslab + g.splits - 1) / g.splits;
+        slab0 = part_id * per;
+        nslab = max(min(nslab - slab0, per), 0);
+    }
     const unsigned fetch_lds = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)wave * (64 * BK * 2));
     // slabs past the end re-fetch the last slab into a stage nobody reads any more
     // the i-th (i < 16) of the loads that bring this wave's part of slab s in
     auto fetch_one = [&](int s, int i) __attribute__((always_inline)) {
-        const unsigned uo = (unsigned)(s < nslab ? s : nslab - 1) * (BK * 2u);
+        const unsigned uo = (unsigned)min(slab0 + max(s < nslab ? s : nslab - 1, 0), g.k / BK - 1) * (BK * 2u);
         const unsigned base = fetch_lds + (unsigned)(s & 1) * DMA_STAGE_BYTES;
         const int j = i >> 1;
         if ((i & 1) == 0) load_to_lds_16(a_rsrc, base + (unsigned)j * (8 * BK * 2), a_off[j], uo);
@@ -575,6 +588,20 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         mfma_step(f1, f0, so_next, 0, s + 2);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
+    if (g.splits > 1) {
+        // partial tile in the accumulation layout: [tile][part][wave][i][j][r][lane] x 16 bytes,
+        // every store instruction 1 KB in a row; the merge kernel reads it the same way
+        f32x4* dst = reinterpret_cast<f32x4*>(g.part) +
+                     ((((int64_t)(logical - g.tile_base) * g.splits + part_id) * 4 + wave) * 64) * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    dst[(i * 16 + j * 4 + r) * 64] = f32x4{acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2], acc[i][j][4 * r + 3]};
+        return;
+    }
     if constexpr (sizeof(TC) == 2) {
         // uniform over the launch: rows of C start on 16 bytes
         if ((g.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(cp) % 16 == 0)) {
@@ -584,6 +611,62 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         }
     }
     store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, l32, h);
+}
+
+// Adds the parts of the k-split tiles in part order and writes C. One thread per 16 bytes of
+// a partial tile: thread (tile, wave, e = 16 i + 4 j + r, lane) owns row
+// 128 (wave / 2) + 32 i + lane % 32 and columns 128 (wave % 2) + 32 j + 8 r + 4 (lane / 32) .. + 4
+// of the tile, as in the four-wave build. Every part's load is sent before the first is used.
+constexpr int kMaxKSplits = 8;
+template <bool F16>
+__global__ void __launch_bounds__(256) gemm_merge_kernel(const GemmArgs g, int c_is_f32) {
+    const int t = (int)blockIdx.x >> 6;
+    const int idx = (((int)blockIdx.x & 63) << 8) + (int)threadIdx.x;
+    const int wave = idx >> 12, e = (idx >> 6) & 63, lane = idx & 63;
+    const f32x4* src = reinterpret_cast<const f32x4*>(g.part) + ((((int64_t)t * g.splits) * 4 + wave) * 64 + e) * 64 + lane;
+    f32x4 v[kMaxKSplits];
+#pragma unroll
+    for (int z = 0; z < kMaxKSplits; z++) {
+        v[z] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (z < g.splits) v[z] = src[(int64_t)z * (4 * 64 * 64)];
+    }
+    f32x4 sum = v[0];
+#pragma unroll
+    for (int z = 1; z < kMaxKSplits; z++)
+        if (z < g.splits) sum += v[z];
+
+    const int tiles_row = g.tiles_n * g.groups;
+    int tm, tn;
+    tile_coords(g.tile_base + t, (g.m + BM - 1) / BM, tiles_row, tm, tn);
+    const int grp = tn / g.tiles_n;
+    tn -= grp * g.tiles_n;
+    void* const cp = grp == 0 ? g.c : g.c_more[grp - 1];
+    const int i = e >> 4, j = (e >> 2) & 3, r = e & 3;
+    const int row = tm * BM + (wave >> 1) * 128 + 32 * i + (lane & 31);
+    const int col = tn * BN + (wave & 1) * 128 + 32 * j + 8 * r + 4 * (lane >> 5);
+    if (row >= g.m) return;
+    if (c_is_f32) {
+        float* dst = reinterpret_cast<float*>(cp) + (int64_t)row * g.ldc + col;
+        if (col + 3 < g.n && g.ldc % 4 == 0 && reinterpret_cast<uintptr_t>(cp) % 16 == 0) {
+            *reinterpret_cast<f32x4*>(dst) = sum;
+        } else {
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+                if (col + jj < g.n) dst[jj] = sum[jj];
+        }
+    } else {
+        u32x2 pk;
+        if constexpr (F16) pk = __builtin_bit_cast(u32x2, __builtin_convertvector(sum, f16x4));
+        else pk = __builtin_bit_cast(u32x2, __builtin_convertvector(sum, bf16x4));
+        unsigned short* dst = reinterpret_cast<unsigned short*>(cp) + (int64_t)row * g.ldc + col;
+        if (col + 3 < g.n && g.ldc % 4 == 0 && reinterpret_cast<uintptr_t>(cp) % 8 == 0) {
+            *reinterpret_cast<u32x2*>(dst) = pk;
+        } else {
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+                if (col + jj < g.n) dst[jj] = (unsigned short)(pk[jj >> 1] >> (16 * (jj & 1)));
+        }
+    }
 }
 
 // Measured on the Klein projections, same box, all with row-by-row stores and row-major tile
@@ -614,7 +697,25 @@ static hipError_t launch_one(const GemmArgs& g0, hipStream_t stream) {
     if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
     if constexpr (!std::is_same<TA, float>::value) {
         if (g_gemm_build == 1 && g.k % BK == 0) {
-            gemm_ring_kernel<F16, TC><<<dim3((unsigned)nwg), dim3(256), kRingLdsBytes, stream>>>(g);
+            // whole tiles first, then (splits > 1) the tiles of the last round in parts, then the merge
+            const int tail = g0.splits > 1 ? g0.tile_base : 0; // the planner leaves the tail size in tile_base
+            if (tail < 0 || tail > nwg || g0.splits > kMaxKSplits || (tail > 0 && g0.part == nullptr)) return hipErrorInvalidValue;
+            g.tile_base = 0;
+            g.splits = 1;
+            const int64_t whole = nwg - tail;
+            if (whole > 0) {
+                gemm_ring_kernel<F16, TC><<<dim3((unsigned)whole), dim3(256), kRingLdsBytes, stream>>>(g);
+                hipError_t e = hipGetLastError();
+                if (e != hipSuccess) return e;
+            }
+            if (tail > 0) {
+                g.tile_base = (int32_t)whole;
+                g.splits = g0.splits;
+                gemm_ring_kernel<F16, TC><<<dim3((unsigned)(tail * g0.splits)), dim3(256), kRingLdsBytes, stream>>>(g);
+                hipError_t e = hipGetLastError();
+                if (e != hipSuccess) return e;
+                gemm_merge_kernel<F16><<<dim3((unsigned)tail * 64u), dim3(256), 0, stream>>>(g, std::is_same<TC, float>::value ? 1 : 0);
+            }
             return hipGetLastError();
         }
         if (g.k % BK == 0) { // whole slabs of 16-bit activations: the direct-to-LDS build
@@ -647,6 +748,30 @@ static hipError_t raise_lds() {
 
 int gemm_tile_rows() { return gemm::BM; }
 int gemm_tile_cols() { return gemm::BN; }
+
+// Only the four-wave build splits (16-bit activations, whole slabs, enough tiles for 256-tiles).
+// A last round that fills at most half the CUs is cut along k so that it fills them: the round
+// then costs 1 / splits of a tile's time plus the partial tiles' trip through memory (256 KB
+// per part, which is why the number of parts is kept small and a fuller round is left whole).
+void gemm_tail_plan(const GemmArgs& g, int a_dtype, int cus, int* tail_tiles, int* splits) {
+    *tail_tiles = 0;
+    *splits = 1;
+    if (a_dtype == kF32 || gemm::g_gemm_build != 1 || g.k % gemm::BK != 0 || cus <= 0) return;
+    const int64_t tiles = (int64_t)((g.m + 255) / 256) * ((g.n + 255) / 256) * g.groups;
+    if (tiles < 160 || tiles > 0x7fffffff) return;
+    const int tail = (int)(tiles % cus);
+    if (tail == 0 || tail * 2 > cus) return;
+    int s = cus / tail;
+    if (s > gemm::kMaxKSplits) s = gemm::kMaxKSplits;
+    const int nslab = g.k / gemm::BK;
+    if (s > nslab / 4) s = nslab / 4; // at least four slabs per part
+    if (s < 2) return;
+    *tail_tiles = tail;
+    *splits = s;
+}
+size_t gemm_part_bytes(int tail_tiles, int splits) {
+    return (size_t)tail_tiles * splits * gemm::BM * gemm::BN * sizeof(float);
+}
 
 hipError_t launch_gemm(const GemmArgs& g, int a_dtype, int w_dtype, int c_dtype, hipStream_t stream) {
     using namespace gemm;

@@ -19,6 +19,13 @@ struct GemmArgs {
     int32_t groups;  // 1..3 products sharing A and every dimension: group i > 0 uses w_more[i-1], c_more[i-1]
     const void* w_more[2];
     void* c_more[2];
+    // Tiles of a partly filled last round, split along k (set by the caller from gemm_tail_plan;
+    // splits <= 1: none). On entry tile_base holds the NUMBER of tail tiles; the launcher runs
+    // the whole tiles first, then the tail tiles in `splits` parts each (fp32 partial tiles to
+    // `part`), then the kernel that adds the parts in part order and writes C.
+    int32_t tile_base;
+    int32_t splits;
+    float* part;
 };
 
 int gemm_tile_rows();
@@ -26,6 +33,11 @@ int gemm_tile_cols();
 // a_dtype: kF32 or the weight's type; w_dtype: kF16 or kBF16; c_dtype: kF32 or the weight's type.
 hipError_t launch_gemm(const GemmArgs& args, int a_dtype, int w_dtype, int c_dtype, hipStream_t stream);
 hipError_t gemm_setup();
+// How launch_gemm would split the last round of this product on a device with `cus` compute
+// units: *tail_tiles tiles in *splits parts each (splits 1: no split), and the bytes of fp32
+// partial tiles that needs.
+void gemm_tail_plan(const GemmArgs& args, int a_dtype, int cus, int* tail_tiles, int* splits);
+size_t gemm_part_bytes(int tail_tiles, int splits);
 void gemm_set_build(int build); // 256-tiles of 16-bit activations: 1 = four-wave build (default), 0 = eight-wave build
 
 } // namespace zdraw

@@ -124,6 +124,7 @@ SYMBOLS = {
     "zdraw_hip_run_gemm_pair": (_int, [_vp, _vp, _vp, _vp, _vp, _GP, _vp, _vp, _GP]),
     "zdraw_hip_run_gemm_triple": (_int, [_vp, _vp, _vp, _vp, _vp, _GP, _vp, _vp, _GP, _vp, _vp, _GP]),
     "zdraw_hip_run_gemm_ext_enc": (_int, [_vp, _vp, _vp, _vp, _GP, _GX]),
+    "zdraw_hip_run_gemm_group_ext_enc": (_int, [_vp, _vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_GP), C.c_uint32, _GX]),
     "zdraw_hip_run_chain_attn_enc": (_int, [_vp, C.POINTER(ChainAttnBuffers), C.POINTER(ChainAttnWeights),
                                             C.POINTER(ChainAttnParams)]),
     "zdraw_hip_mfma_probe": (_int, [_int, _int, C.POINTER(C.c_double)]),
@@ -138,6 +139,7 @@ SYMBOLS = {
     "zdraw_hip_set_attention_variant": (None, [_int]),
     "zdraw_hip_set_gemm_build": (None, [_int]),
     "zdraw_hip_attention_tail_plan": (None, [_u64, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "zdraw_hip_gemm_tail_plan": (None, [_u32, _u32, _u32, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "zdraw_hip_abi_sizeof": (_sz, [_int]),
     "zdraw_hip_last_error": (C.c_char_p, []),
 }
