@@ -57,7 +57,9 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
     // One wait for everything: the stores below sit under a predicate, and past a branch the
     // compiler no longer knows how many stores are younger than a load it waits for, so it
     // would wait for the previous heads' stores as well.
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    // (Z-Image only: its coefficients are the last load to come back anyway. Klein's heads are
+    // worked on as their rows arrive, which measured 5 % faster than one wait.)
+    if constexpr (MODE != kQkKlein) __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
     // the token's weights and rope row stay in registers across its heads
     f32x4 w0, w1;
     if (w_f32) {
