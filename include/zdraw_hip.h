@@ -66,7 +66,9 @@ enum {
 /* Where norm+rope happens for the fused entry. */
 enum {
     ZDRAW_HIP_K_IN_TILE_LOAD = 0, /* inside the attention kernel: Q in its prologue, K per tile */
-    ZDRAW_HIP_K_PREPASS = 1       /* one pre-pass kernel prepares Q and K into library scratch, then attention */
+    ZDRAW_HIP_K_PREPASS = 1       /* one pre-pass kernel prepares Q and K as bf16 in library scratch (f32 operands:
+                                   * the same launch also rounds V, as krms_rope_hm / to_headmajor_f16 write half
+                                   * copies, zflux2_glue_shader.zig:95-122), then attention on 16-bit rows */
 };
 
 /*

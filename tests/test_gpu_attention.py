@@ -189,6 +189,27 @@ def test_small_configs_all_rows(ctx, name, k_site, dtype, bounded):
     assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
 
 
+@pytest.mark.parametrize("name", ["klein_512_x4", "zimage_1024", "klein_edit_ragged"])
+def test_f32_operands_are_rounded_once_and_take_the_16_bit_kernel(ctx, name):
+    # With the pre-pass, f32 Q, K and V are rounded to bf16 on their way into scratch and the
+    # attention kernel is the one that runs on bf16 operands. Operands that are bf16 values
+    # held as f32 must therefore give the same bits as the same values handed over as bf16.
+    w = wl.by_name(name, seed=8, small=True)
+    for f in ("q", "k", "v"):
+        setattr(w, f, host.bf16_bits_to_f32(host.f32_to_bf16_bits(getattr(w, f))))
+    outs = []
+    for dtype in (hip.F32, hip.BF16):
+        res = wl.Resident(ctx, w, dtype=dtype, k_site=hip.K_PREPASS)
+        res.ext.out_dtype = hip.BF16
+        rc = hip.lib().zdraw_hip_run_attention_fused(ctx.queue, res.q.handle, res.k.handle, res.v.handle, res.o.handle,
+                                                     C.byref(res.params), C.byref(res.ext), C.byref(res.ops))
+        assert rc == 0, hip.last_error()
+        outs.append(host.bf16_bits_to_f32(res.o.read(np.uint16, (w.batch, w.tokens, w.heads, 128))))
+        res.release()
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    refimpl.check_close(outs[0], refimpl.reference_rows(w), name)
+
+
 # ------------------------------------- configs 2-5, full size, sampled rows
 FULL = [("klein_1024", 48), ("klein_512_x4", 40), ("zimage_1024", 40), ("klein_edit_ragged", 28)]
 

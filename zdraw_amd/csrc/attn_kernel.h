@@ -84,7 +84,7 @@ struct PrepArgs {
     int64_t x_bs, x_ts, x_hs;
     int64_t y_bs, y_ts, y_hs;
     int32_t tokens, heads, batch;
-    int32_t mode;       // QkMode (never kQkNone)
+    int32_t mode;       // QkMode; kQkNone = the rows are only rounded and re-laid (V beside a prepared Q and K)
     int32_t out_dtype;  // kF32 or kBF16
     float scale;        // multiplies the result (1 for K; log2(e)/sqrt(head_dim) when Q is prepared for attention)
     QkOps qk;
@@ -95,7 +95,9 @@ struct PrepArgs {
 };
 
 struct PrepPair {
-    PrepArgs op[2];
+    PrepArgs op[3]; // Q, K and, when the launch has a third operand, rows that are only rounded (mode kQkNone)
+    int32_t count;
+    int32_t pad0;
 };
 
 // Kernel shape: 0 = 8 waves x 32 query rows (one workgroup per CU, 8-stage LDS

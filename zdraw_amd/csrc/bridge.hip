@@ -173,6 +173,9 @@ struct FusedPlan {
     bool prepass;
     PrepArgs prep;   // K pre-pass
     PrepArgs prep_q; // Q pre-pass (same launch condition)
+    PrepArgs prep_v; // f32 operands only: V rounded to bf16 by the same launch
+    bool round_v = false;
+    int prep_in_dtype = kF32; // element type the pre-pass reads
     int w_dtype = kF32; // element type of the norm weights (16-bit only with the pre-pass)
 };
 
@@ -340,11 +343,17 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     plan->prepass = false;
     if (x->qk_mode != ZDRAW_HIP_QK_NONE && x->k_site == ZDRAW_HIP_K_PREPASS) {
         // Q and K are normalised and rotated once into scratch slots 0 and 1, head-major,
-        // in the activation dtype; the attention kernel then reads them as they are. One
+        // as bf16; the attention kernel then reads them as they are. One
         // pass over the rows reads a token's rope row once for all its heads; inside the
         // attention kernel every (head, query block) workgroup would fetch its own copy.
         // Q also takes the softmax scale (in the exp2 domain) here, before the rounding.
-        const size_t es = elem_size(x->in_dtype);
+        // f32 operands (the reference's resident layout, zflux2_resident.zig:1642-1669, writes
+        // half-precision head-major copies the same way): the pre-pass rounds Q and K to bf16
+        // and the same launch rounds V into slot 2, so the attention kernel runs its
+        // direct-to-LDS build on 16-bit rows instead of rounding every block it loads.
+        const bool to_bf16 = x->in_dtype == ZDRAW_HIP_F32;
+        const uint32_t prep_out = to_bf16 ? (uint32_t)ZDRAW_HIP_BF16 : x->in_dtype;
+        const size_t es = elem_size(prep_out);
         const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * es;
         Buffer* sq = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 0, bytes));
         Buffer* sk = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 1, bytes));
@@ -359,7 +368,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         pr.y_hs = (int64_t)p->tokens * kHeadDim;
         pr.tokens = a.tokens; pr.heads = a.heads; pr.batch = a.batch;
         pr.mode = (int32_t)x->qk_mode;
-        pr.out_dtype = (int32_t)x->in_dtype;
+        pr.out_dtype = (int32_t)prep_out;
         pr.qk = a.qk;
         pr.w_dtype = plan->w_dtype;
         PrepArgs pq = pr;
@@ -385,6 +394,26 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         plan->args.q_bs = pr.y_bs; plan->args.q_ts = pr.y_ts; plan->args.q_hs = pr.y_hs;
         plan->args.q_mode = kQkNone;
         plan->args.scale_log2 = 1.0f;
+        plan->prep_in_dtype = (int)x->in_dtype;
+        if (to_bf16) {
+            Buffer* sv = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 2, bytes));
+            if (!sv) {
+                set_err("scratch allocation failed");
+                return ZDRAW_HIP_ERR_HANDLE;
+            }
+            PrepArgs pv = pr;
+            pv.mode = kQkNone;
+            pv.x = a.v;
+            pv.y = sv->ptr;
+            pv.x_bs = a.v_bs; pv.x_ts = a.v_ts; pv.x_hs = a.v_hs;
+            pv.w = pv.w_txt = nullptr;
+            pv.scale = 1.0f;
+            plan->prep_v = pv;
+            plan->round_v = true;
+            plan->args.v = sv->ptr;
+            plan->args.v_bs = pr.y_bs; plan->args.v_ts = pr.y_ts; plan->args.v_hs = pr.y_hs;
+            plan->in_dtype = kBF16;
+        }
     }
     return ZDRAW_HIP_OK;
 }
@@ -399,8 +428,8 @@ int enqueue(const FusedPlan& plan, hipStream_t stream) {
         g_setup_done = true;
     }
     if (plan.prepass) {
-        const PrepArgs both[2] = {plan.prep_q, plan.prep};
-        hipError_t e = launch_qk_prepass(both, 2, plan.in_dtype, stream);
+        const PrepArgs ops[3] = {plan.prep_q, plan.prep, plan.prep_v};
+        hipError_t e = launch_qk_prepass(ops, plan.round_v ? 3 : 2, plan.prep_in_dtype, stream);
         if (e != hipSuccess) {
             set_err("qk pre-pass launch: %s", hipGetErrorString(e));
             return ZDRAW_HIP_ERR_HANDLE;

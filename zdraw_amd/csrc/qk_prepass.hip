@@ -24,7 +24,7 @@ constexpr int kPrepTokens = 4; // tokens (waves) per workgroup
 template <typename TIn, int MODE, int G>
 __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const PrepPair pair) {
     // grid z = operand * batch + segment; the choice is uniform over the workgroup
-    const int op = (int)blockIdx.z >= pair.op[0].batch ? 1 : 0;
+    const int op = (int)blockIdx.z / pair.op[0].batch;
     const PrepArgs& p = pair.op[op];
     const int tok_raw = (int)blockIdx.x * kPrepTokens + (int)(threadIdx.x >> 6);
     const bool tok_ok = tok_raw < p.tokens;
@@ -35,6 +35,34 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
     // Every load of the lane is issued before the first is used, with clamped addresses
     // instead of predicates: no branch, so nothing waits for an earlier load to come back
     // before the next is sent.
+    if (p.mode == kQkNone) {
+        // rows that are only rounded and re-laid (V beside a prepared Q and K)
+        const TIn* src = reinterpret_cast<const TIn*>(p.x) + (int64_t)seg * p.x_bs + (int64_t)tok * p.x_ts + d0;
+        Raw8<TIn> raw[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const int head = h0 + 4 * g;
+            raw[g] = ld_raw8<TIn>(src + (int64_t)(head < p.heads ? head : p.heads - 1) * p.x_hs, true);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0), once: see below
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const int head = h0 + 4 * g;
+            float x[8];
+            unpack8(raw[g], x);
+            if (tok_ok && head < p.heads) {
+                const int64_t off = (int64_t)seg * p.y_bs + (int64_t)tok * p.y_ts + (int64_t)head * p.y_hs + d0;
+                if (p.out_dtype == kF32) {
+                    float* dst = reinterpret_cast<float*>(p.y) + off;
+                    *reinterpret_cast<f32x4*>(dst) = f32x4{x[0], x[1], x[2], x[3]};
+                    *reinterpret_cast<f32x4*>(dst + 4) = f32x4{x[4], x[5], x[6], x[7]};
+                } else {
+                    *reinterpret_cast<u32x4*>(reinterpret_cast<bf16_t*>(p.y) + off) = pack_bf16x8(x);
+                }
+            }
+        }
+        return;
+    }
     // Order of the loads: the token's position (Z-Image) first, because the address of its
     // rope coefficients depends on it and loads come back in the order they were sent; then
     // the norm weights, the rows, the rope coefficients. Nothing is used before all are sent.
@@ -109,17 +137,20 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
     }
 }
 
-// One launch covers `count` operands (1 or 2) of equal tokens/heads/batch/mode.
+// One launch covers `count` operands (1 to 3) of equal tokens/heads/batch: the first two are
+// normalised and rotated (same mode), a third is only rounded and re-laid (mode kQkNone).
 hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipStream_t stream) {
-    if (count < 1 || count > 2) return hipErrorInvalidValue;
+    if (count < 1 || count > 3) return hipErrorInvalidValue;
     const PrepArgs& p = ops[0];
     if (p.batch <= 0 || p.heads <= 0 || p.tokens <= 0 || p.batch * count > 65535) return hipErrorInvalidValue;
-    if (count == 2 && (ops[1].batch != p.batch || ops[1].heads != p.heads || ops[1].tokens != p.tokens ||
-                       ops[1].mode != p.mode || ops[1].out_dtype != p.out_dtype))
-        return hipErrorInvalidValue;
+    for (int i = 1; i < count; i++) {
+        if (ops[i].batch != p.batch || ops[i].heads != p.heads || ops[i].tokens != p.tokens) return hipErrorInvalidValue;
+        if (ops[i].mode != (i == 2 ? (int32_t)kQkNone : p.mode)) return hipErrorInvalidValue;
+    }
     PrepPair pair;
-    pair.op[0] = ops[0];
-    pair.op[1] = ops[count - 1];
+    for (int i = 0; i < 3; i++) pair.op[i] = ops[i < count ? i : count - 1];
+    pair.count = count;
+    pair.pad0 = 0;
     const bool wide_pass = (p.heads + 31) / 32 < (p.heads + 23) / 24; // fewer passes over the heads with 32 per pass
     const int per_pass = wide_pass ? 32 : 24;
     const dim3 grid((unsigned)((p.tokens + kPrepTokens - 1) / kPrepTokens), (unsigned)((p.heads + per_pass - 1) / per_pass),
