@@ -304,8 +304,9 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
 
 /* ---- library-owned scratch (metal_c.zig:321-325) -------------------------- */
 /* Grow-only, process-lifetime, filled at (re)allocation with 0x00 (0xFF when
- * ZDRAW_SCRATCH_POISON is set, metal_api.m:6147-6181). slot in [0, 6): 0-2 prepared
- * operands, 3-4 the parts of key-split attention tiles, 5 the parts of k-split GEMM tiles. */
+ * ZDRAW_SCRATCH_POISON is set, metal_api.m:6147-6181). slot in [0, 7): 0-2 prepared
+ * operands, 3-4 the parts of key-split attention tiles, 5 the parts of k-split GEMM tiles,
+ * 6 a GEMM's f32 activations rounded to 16 bits. */
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes);
 
 /* ---- counters and timing (metal_api.m:333-353, 420-433) ------------------- */

@@ -462,7 +462,8 @@ def test_scratch_is_grow_only_and_filled(ctx):
     c = L.zdraw_hip_attn_scratch(ctx.device, 4, want + (1 << 20))
     assert L.zdraw_hip_buffer_length(c) >= want + (1 << 20)
     assert L.zdraw_hip_attn_scratch(ctx.device, 5, 16)      # the k-split GEMM tiles' parts
-    assert not L.zdraw_hip_attn_scratch(ctx.device, 6, 16)  # past the last slot
+    assert L.zdraw_hip_attn_scratch(ctx.device, 6, 16)      # a GEMM's rounded f32 activations
+    assert not L.zdraw_hip_attn_scratch(ctx.device, 7, 16)  # past the last slot
 
 
 # --------------------------------------------- standalone QK-norm + rope (mqk.run)

@@ -313,14 +313,16 @@ def test_pair_and_triple_of_one_activation(ctx, pipe, count, same_shape):
         b.release()
 
 
+@pytest.mark.parametrize("a32", [False, True])
 @pytest.mark.parametrize("c_dtype", [hip.F32, hip.BF16])
 @pytest.mark.parametrize("build", [1, 0])
-def test_many_tile_problem_runs_the_256_tile_builds(ctx, build, c_dtype):
+def test_many_tile_problem_runs_the_256_tile_builds(ctx, build, c_dtype, a32):
     # 13 x 13 = 169 tiles of 256 x 256 (ragged last row and column of tiles): enough tiles for
     # the 256-tile builds (four waves by default, eight behind the knob), which the small
     # shapes above never reach; with 16-bit C the interior tiles leave through LDS as whole
     # rows and the edge tiles element by element. Against the oracle on identically rounded
-    # operands.
+    # operands. a32: f32 activations, which are rounded once into scratch ahead of the product
+    # and then take the same builds.
     L = hip.lib()
     rng = np.random.default_rng(23)
     m, k, n = 3300, 128, 3290
@@ -331,7 +333,7 @@ def test_many_tile_problem_runs_the_256_tile_builds(ctx, build, c_dtype):
     w_bits, wr = to16(w, hip.W_BF16)
     L.zdraw_hip_set_gemm_build(build)
     try:
-        raw = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, c_dtype, ldc=ldc,
+        raw = run_ext(ctx, a if a32 else a_bits, w_bits, m, k, n, hip.W_BF16, hip.F32 if a32 else hip.BF16, c_dtype, ldc=ldc,
                       c_init=np.zeros(m * ldc * (4 if c_dtype == hip.F32 else 2), np.uint8))
     finally:
         L.zdraw_hip_set_gemm_build(1)

@@ -580,7 +580,7 @@ int finish_blocking(Queue* qu, hipEvent_t start, hipEvent_t stop) {
     return ZDRAW_HIP_OK;
 }
 
-Buffer* g_scratch[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+Buffer* g_scratch[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 
 bool scratch_poisoned(int slot) {
     // ZDRAW_SCRATCH_POISON: "1" every slot, "attn" the group, "attn:2" one slot
@@ -654,11 +654,23 @@ int enqueue_gemm_group(void* a, void* const* ws, void* const* cs, const uint64_t
     g.tiles_n = (int32_t)((p->n + (uint32_t)gemm_tile_cols() - 1) / (uint32_t)gemm_tile_cols());
     if ((uint64_t)g.tiles_n * (uint64_t)groups * ((p->m + (uint32_t)gemm_tile_rows() - 1) / (uint32_t)gemm_tile_rows()) > 0x7fffffffull)
         return unavailable("grid too large");
+    int a_eff = (int)x->a_dtype;
+    if (const size_t rb = gemm_round_bytes(g, (int)x->a_dtype)) {
+        // f32 activations are rounded to the weight's type once, into scratch slot 6, and the
+        // product then runs as for 16-bit activations
+        Buffer* a16 = static_cast<Buffer*>(zdraw_hip_attn_scratch(queue->dev, 6, rb));
+        if (!a16) {
+            set_err("scratch allocation failed");
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        g.a16 = a16->ptr;
+        a_eff = (int)wt;
+    }
     {
         // a last round of tiles that fills at most half the CUs runs split along k; its fp32
         // partial tiles go through scratch slot 5
         int tail = 0, splits = 1;
-        gemm_tail_plan(g, (int)x->a_dtype, queue->dev->cus, &tail, &splits);
+        gemm_tail_plan(g, a_eff, queue->dev->cus, &tail, &splits);
         if (splits > 1) {
             Buffer* part = static_cast<Buffer*>(zdraw_hip_attn_scratch(queue->dev, 5, gemm_part_bytes(tail, splits)));
             if (!part) {
@@ -1195,7 +1207,7 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
 
 // ------------------------------------------------------------------ scratch
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes) {
-    if (!device || slot < 0 || slot >= 6 || bytes == 0) return nullptr;
+    if (!device || slot < 0 || slot >= 7 || bytes == 0) return nullptr;
     Buffer* cur = g_scratch[slot];
     if (cur && cur->len >= bytes) return cur;
     // Grow: work already enqueued may still read the old allocation, so drain

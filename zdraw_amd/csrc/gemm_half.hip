@@ -669,6 +669,37 @@ __global__ void __launch_bounds__(256) gemm_merge_kernel(const GemmArgs g, int c
     }
 }
 
+// f32 activations rounded to the weight's 16-bit type, once, into dense [m][k] rows: the
+// products that follow then move their A slabs straight into LDS like 16-bit activations
+// instead of rounding every slab of every tile (each row of A is read by every column tile).
+template <bool F16>
+__global__ void __launch_bounds__(256) gemm_round_kernel(const float* a, int64_t lda, unsigned short* out, int m, int k) {
+    // grid x = row, grid y = 4096-element stretch of the row; a thread rounds two groups of 8
+    const int row = (int)blockIdx.x;
+    const int c0 = (int)blockIdx.y * 4096 + (int)threadIdx.x * 8;
+    const float* src = a + (int64_t)row * lda;
+    unsigned short* dst = out + (int64_t)row * k;
+    f32x4 lo[2], hi[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int c = min(c0 + u * 2048, k - 8); // past the end: re-read the last group, not stored
+        lo[u] = *reinterpret_cast<const f32x4*>(src + c);
+        hi[u] = *reinterpret_cast<const f32x4*>(src + c + 4);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int c = c0 + u * 2048;
+        if (c >= k) continue;
+        f32x8 v;
+#pragma unroll
+        for (int i = 0; i < 4; i++) { v[i] = lo[u][i]; v[4 + i] = hi[u][i]; }
+        u32x4 r;
+        if constexpr (F16) r = __builtin_bit_cast(u32x4, __builtin_convertvector(v, f16x8));
+        else r = __builtin_bit_cast(u32x4, __builtin_convertvector(v, bf16x8));
+        *reinterpret_cast<u32x4*>(dst + c) = r;
+    }
+}
+
 // Measured on the Klein projections, same box, all with row-by-row stores and row-major tile
 // order: eight waves (two per SIMD, 64 x 128 each) 1048-1217 TFLOP/s; four waves with the
 // schedule above 1047-1248; four waves with the simple loop of the eight-wave build 960-1120.
@@ -773,9 +804,31 @@ size_t gemm_part_bytes(int tail_tiles, int splits) {
     return (size_t)tail_tiles * splits * gemm::BM * gemm::BN * sizeof(float);
 }
 
-hipError_t launch_gemm(const GemmArgs& g, int a_dtype, int w_dtype, int c_dtype, hipStream_t stream) {
+size_t gemm_round_bytes(const GemmArgs& g, int a_dtype) {
+    // Whole slabs (the direct-to-LDS builds need them) and at least one full tile each way. The
+    // pass moves 6 bytes per element of A through memory; measured at 4608 rows it pays at every
+    // shape tried (n = 9216: 0.268 -> 0.263 ms with f32 C; k = 12288, n = 3072: 0.384 -> 0.372;
+    // k = n = 3840: 0.225 -> 0.155, where it also opens the way to the k-split last round).
+    if (a_dtype != kF32 || g.k % gemm::BK != 0 || g.m < 256 || g.n < 256) return 0;
+    return (size_t)g.m * (size_t)g.k * 2;
+}
+
+hipError_t launch_gemm(const GemmArgs& g0, int a_dtype, int w_dtype, int c_dtype, hipStream_t stream) {
     using namespace gemm;
     typedef unsigned short h16; // a 16-bit operand in the compute type (bf16 or f16 per the weight)
+    GemmArgs g = g0;
+    if (a_dtype == kF32 && g.a16 != nullptr && gemm_round_bytes(g, a_dtype) != 0) {
+        const dim3 grid((unsigned)g.m, (unsigned)((g.k + 4095) / 4096));
+        if (w_dtype == kF16)
+            gemm_round_kernel<true><<<grid, dim3(256), 0, stream>>>(static_cast<const float*>(g.a), g.lda, static_cast<h16*>(g.a16), g.m, g.k);
+        else
+            gemm_round_kernel<false><<<grid, dim3(256), 0, stream>>>(static_cast<const float*>(g.a), g.lda, static_cast<h16*>(g.a16), g.m, g.k);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        g.a = g.a16;
+        g.lda = g.k;
+        a_dtype = w_dtype;
+    }
     if (w_dtype == kBF16) {
         if (a_dtype == kF32 && c_dtype == kF32) return launch_one<float, false, float>(g, stream);
         if (a_dtype == kF32 && c_dtype == kBF16) return launch_one<float, false, h16>(g, stream);

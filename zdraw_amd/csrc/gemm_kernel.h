@@ -26,6 +26,9 @@ struct GemmArgs {
     int32_t tile_base;
     int32_t splits;
     float* part;
+    // f32 activations: room for A rounded to the weight's type, [m][k] 16-bit (gemm_round_bytes
+    // says how much; null: A is rounded block by block on its way into LDS instead)
+    void* a16;
 };
 
 int gemm_tile_rows();
@@ -38,6 +41,9 @@ hipError_t gemm_setup();
 // partial tiles that needs.
 void gemm_tail_plan(const GemmArgs& args, int a_dtype, int cus, int* tail_tiles, int* splits);
 size_t gemm_part_bytes(int tail_tiles, int splits);
+// Bytes of scratch launch_gemm wants for rounding f32 activations once, ahead of the product
+// (0: not worth it or not possible for this shape).
+size_t gemm_round_bytes(const GemmArgs& args, int a_dtype);
 void gemm_set_build(int build); // 256-tiles of 16-bit activations: 1 = four-wave build (default), 0 = eight-wave build
 
 } // namespace zdraw
