@@ -195,8 +195,9 @@ def chain_main(args):
     bits = lambda a: host.f32_to_bf16_bits(a)
     x = rng.standard_normal((tokens, hidden), dtype=np.float32)
     wall_w = rng.standard_normal((4, inner, hidden), dtype=np.float32) * np.float32(hidden ** -0.5)
-    nb, wb = ctx.buffer(bits(x)), ctx.buffer(bits(wall_w))
-    qb, kb, vb, mixb, ob = (ctx.buffer(nbytes=tokens * inner * 2) for _ in range(5))
+    act32 = args.chain_act == "f32"
+    nb, wb = ctx.buffer(x if act32 else bits(x)), ctx.buffer(bits(wall_w))
+    qb, kb, vb, mixb, ob = (ctx.buffer(nbytes=tokens * inner * (4 if act32 else 2)) for _ in range(5))
     ones = ctx.buffer(np.ones(128, np.float32))
     posb = ctx.buffer(np.ascontiguousarray(w.pos, dtype=np.uint64))
     ropeb = ctx.buffer(w.rope_pairs)
@@ -206,7 +207,7 @@ def chain_main(args):
     p.qk = hip.QkNormParams(tokens, heads, heads, 128, hip.W_F32, hip.W_F32, *wl.ZIMAGE_DIMS, wl.ZIMAGE_EPS, 0, 0,
                             *w.rope_bases)
     p.attn = hip.AttnParams(tokens, heads, heads, 128, 0, 0)
-    p.act_dtype = hip.BF16
+    p.act_dtype = hip.F32 if act32 else hip.BF16
     p.score_bound = host.score_bound(np.ones(128, np.float32), np.ones(128, np.float32), None, None)
     bufs = hip.ChainAttnBuffers(nb.handle, qb.handle, kb.handle, vb.handle, mixb.handle, ob.handle)
     wts = hip.ChainAttnWeights(wb.handle, wb.handle, wb.handle, ones.handle, ones.handle, posb.handle, ropeb.handle,
@@ -236,7 +237,7 @@ def chain_main(args):
     L.zdraw_hip_event_sync(e1)
     wall = time.perf_counter() - t0
     dev_ms = L.zdraw_hip_event_elapsed_ms(e0, e1) / args.steps
-    out = host.bf16_bits_to_f32(ob.read(np.uint16, (tokens, hidden)))
+    out = ob.read(np.float32, (tokens, hidden)) if act32 else host.bf16_bits_to_f32(ob.read(np.uint16, (tokens, hidden)))
     if not np.isfinite(out).all():
         raise RuntimeError("non-finite output")
     gemm_flops = 4 * 2.0 * tokens * hidden * inner
@@ -248,7 +249,7 @@ def chain_main(args):
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"zimage chain segment: tokens {tokens}, heads {heads}, hidden {hidden}, bf16 activations and weights",
+        "config": {"workload": f"zimage chain segment: tokens {tokens}, heads {heads}, hidden {hidden}, {args.chain_act} activations, bf16 weights",
                    "gemm_gflop": gemm_flops / 1e9, "attention_gflop": attn_flops / 1e9,
                    "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS, "untimed_spinup_segments": spun},
         "roofline": {"bound": "mfma", "achieved": flops / (dev_ms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
@@ -351,6 +352,8 @@ def main():
     ap.add_argument("--path", choices=["attention", "gemm", "chain", "wide"], default="attention",
                     help="attention (the headline metric) or the projection GEMM beside it")
     ap.add_argument("--wide-tokens", type=int, default=16384, help="--path wide: sequence length (multiple of 64)")
+    ap.add_argument("--chain-act", choices=["bf16", "f32"], default="bf16",
+                    help="--path chain: activation buffers as bf16, or f32 as the reference's chain keeps them")
     ap.add_argument("--m", type=int, default=4608)
     ap.add_argument("--k", type=int, default=3072)
     ap.add_argument("--n", type=int, default=9216)
