@@ -46,7 +46,10 @@ namespace fwd {
 #define ZDRAW_READ_BATCH 2    // slots whose fragment reads are issued together (one wait per batch)
 #endif
 #ifndef ZDRAW_MFMA_PRIO
-#define ZDRAW_MFMA_PRIO 1     // wave priority while an MFMA is issued (0 = leave it alone)
+#define ZDRAW_MFMA_PRIO 1     // wave priority while an MFMA is issued, builds that stage blocks through registers (0 = leave it alone)
+#endif
+#ifndef ZDRAW_MFMA_PRIO_DIRECT
+#define ZDRAW_MFMA_PRIO_DIRECT 0 // the same for the direct-to-LDS build
 #endif
 #ifndef ZDRAW_DIRECT_LDS
 #define ZDRAW_DIRECT_LDS 1    // prepared bf16 K/V blocks go from global memory straight into LDS
@@ -129,7 +132,11 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     constexpr int AHEAD = NST == 8 ? (DMA ? 5 : 4) : 2;
     constexpr int LA = ZDRAW_LDS_LOOKAHEAD;   // slots between an LDS fragment read and its MFMA
     constexpr int RB = ZDRAW_READ_BATCH;      // slots whose reads are issued together (divides 16 and LA)
-    constexpr int MFMA_PRIO = ZDRAW_MFMA_PRIO; // wave priority while an MFMA is being issued
+    // Wave priority while an MFMA is being issued. The register-staged builds gain from it (the
+    // masked one loses 13 % without). The direct-to-LDS build runs 5 % fewer cycles per
+    // workgroup without the two s_setprio per MFMA; the chip sits on its power limit, so the
+    // clock gives part of that back and 2 % is left.
+    constexpr int MFMA_PRIO = DMA ? ZDRAW_MFMA_PRIO_DIRECT : ZDRAW_MFMA_PRIO;
     constexpr int STORE_SLOT = ZDRAW_STORE_SLOT; // slot after which the ring store is issued
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* const Ks = reinterpret_cast<bf16_t*>(smem);
