@@ -219,9 +219,7 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int g = 0; g < 8; g++) {
-            __builtin_amdgcn_s_setprio(1);
             sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[g], qf[g], sp, 0, 0, 0);
-            __builtin_amdgcn_s_setprio(0);
             // softmax of block b in the exp2 domain (the scale rides on Q) with a lazy maximum:
             // the reference point moves only when this block's maximum exceeds it by more than kTau
             if (g == 0) {
@@ -262,9 +260,7 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
 #pragma unroll
         for (int idx = 0; idx < 8; idx++) {
             const bf16x8 vf = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(vlo[idx], vhi[idx], 0, 1, 2, 3, 4, 5, 6, 7));
-            __builtin_amdgcn_s_setprio(1);
             oacc[idx & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, idx < 4 ? p0 : p1, oacc[idx & 3], 0, 0, 0);
-            __builtin_amdgcn_s_setprio(0);
             if (idx == 1) x_write(sp); // the S MFMAs have drained by now
             __builtin_amdgcn_sched_barrier(0);
         }

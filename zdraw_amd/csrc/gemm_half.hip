@@ -558,9 +558,7 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         for (int t = 0; t < 16; t++) {
             if (fetch >= 0) fetch_one(fetch, t);
             if (t < 8) read_one(nxt, nxt_stage_off, nxt_kk, t);
-            __builtin_amdgcn_s_setprio(1);
             acc[t >> 2][t & 3] = mfma<F16>(cur.w[t & 3], cur.a[t >> 2], acc[t >> 2][t & 3]);
-            __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
