@@ -175,3 +175,73 @@ def test_chain_attention_segment_refuses_what_it_cannot_run(ctx):
     assert L.zdraw_hip_batch_end(batch) == 0
     for b in (z, w, nw, posb, ropeb):
         b.release()
+
+
+def test_full_size_segment_rerun_builds_and_exact_scaling(ctx):
+    # The zimage_1024 shape (4608 tokens, 30 heads, hidden 3840, bf16): the q/k/v group is 810
+    # tiles and the output projection 270, so both run their last round split along k. No CPU
+    # oracle finishes this size; what the domain fixes instead: a rerun gives the same bits;
+    # the eight-wave GEMM build, which never splits, gives the same values up to the order of
+    # the fp32 sums; doubling the projection weights (exact in bf16) doubles every output bit
+    # for bit; and f32 activation buffers holding the same bf16 values agree to rounding.
+    L = hip.lib()
+    w = wl.by_name("zimage_1024", seed=3)
+    tokens, heads = w.tokens, w.heads
+    hidden = inner = heads * 128
+    for m_, k_, n_, g_, want in ((tokens, hidden, inner, 3, (42, 6)), (tokens, inner, hidden, 1, (14, 8))):
+        t, s = C.c_uint32(), C.c_uint32()
+        L.zdraw_hip_gemm_tail_plan(m_, k_, n_, g_, 256, C.byref(t), C.byref(s))
+        assert (t.value, s.value) == want
+    rng = np.random.default_rng(3)
+    x = host.bf16_bits_to_f32(host.f32_to_bf16_bits(rng.standard_normal((tokens, hidden), dtype=np.float32)))
+    wall = rng.standard_normal((4, inner, hidden), dtype=np.float32) * np.float32(hidden ** -0.5)
+    wall2 = wall.copy()
+    wall2[3] *= 2.0
+    ones = ctx.buffer(np.ones(128, np.float32))
+    posb = ctx.buffer(np.ascontiguousarray(w.pos, dtype=np.uint64))
+    ropeb = ctx.buffer(w.rope_pairs)
+
+    def run(act, weights, build=1):
+        esz = 4 if act == hip.F32 else 2
+        nb = ctx.buffer(x if act == hip.F32 else host.f32_to_bf16_bits(x))
+        wb = ctx.buffer(host.f32_to_bf16_bits(weights))
+        qb, kb, vb, mixb, ob = (ctx.buffer(nbytes=tokens * inner * esz) for _ in range(5))
+        p = hip.ChainAttnParams()
+        for i, name in enumerate(("q", "k", "v", "proj")):
+            setattr(p, name, hip.GemmParams(tokens, hidden, inner, hip.W_BF16, hip.GEMM_HALF, i * inner * hidden * 2))
+        p.qk = hip.QkNormParams(tokens, heads, heads, 128, hip.W_F32, hip.W_F32, *wl.ZIMAGE_DIMS, wl.ZIMAGE_EPS, 0, 0,
+                                *w.rope_bases)
+        p.attn = hip.AttnParams(tokens, heads, heads, 128, 0, 0)
+        p.act_dtype = act
+        p.score_bound = host.score_bound(np.ones(128, np.float32), np.ones(128, np.float32), None, None)
+        bufs = hip.ChainAttnBuffers(nb.handle, qb.handle, kb.handle, vb.handle, mixb.handle, ob.handle)
+        wts = hip.ChainAttnWeights(wb.handle, wb.handle, wb.handle, ones.handle, ones.handle, posb.handle, ropeb.handle,
+                                   wb.handle)
+        L.zdraw_hip_set_gemm_build(build)
+        try:
+            batch = L.zdraw_hip_batch_begin(ctx.queue)
+            rc = L.zdraw_hip_run_chain_attn_enc(batch, C.byref(bufs), C.byref(wts), C.byref(p))
+            assert L.zdraw_hip_batch_end(batch) == 0
+        finally:
+            L.zdraw_hip_set_gemm_build(1)
+        assert rc == 0, hip.last_error()
+        out = ob.read(np.float32, (tokens, hidden)) if act == hip.F32 else host.bf16_bits_to_f32(ob.read(np.uint16, (tokens, hidden)))
+        for b in (nb, wb, qb, kb, vb, mixb, ob):
+            b.release()
+        return out
+
+    base = run(hip.BF16, wall)
+    assert np.isfinite(base).all() and np.abs(base).max() > 0
+    assert np.array_equal(base.view(np.uint32), run(hip.BF16, wall).view(np.uint32))
+    assert np.array_equal((2.0 * base).view(np.uint32), run(hip.BF16, wall2).view(np.uint32))
+    scale = float(np.sqrt(np.mean(base.astype(np.float64) ** 2)))
+    whole = run(hip.BF16, wall, build=0)
+    err = np.abs(base - whole)
+    assert err.max() <= 2e-2 * scale and err.mean() <= 2e-3 * scale, (err.max(), err.mean(), scale)
+    # f32 buffers keep q, k, v and the attention output unrounded between the steps: four bf16
+    # hand-over roundings apart, so half a percent of the output's scale on average
+    f32 = run(hip.F32, wall)
+    err = np.abs(base - f32)
+    assert err.max() <= 1e-1 * scale and err.mean() <= 1e-2 * scale, (err.max(), err.mean(), scale)
+    for b in (ones, posb, ropeb):
+        b.release()
