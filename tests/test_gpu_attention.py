@@ -112,6 +112,27 @@ def test_block_cases_match_cpu(ctx, tokens, heads):
     assert np.array_equal(got.view(np.uint32), pooled.view(np.uint32))
 
 
+@pytest.mark.parametrize("tokens,heads,valid", [(1024, 2, None), (1100, 3, None), (1100, 2, 1000), (1056, 1, 37)])
+def test_long_plain_f32_rows_are_rounded_once_ahead_of_the_kernel(ctx, tokens, heads, valid):
+    # from 1024 tokens on, plain attention on f32 rows rounds Q (with the softmax scale), K and
+    # V to bf16 into scratch with one launch and runs the kernel for 16-bit rows; same contract
+    # and tolerance as the short cases, ragged last block and key limit included
+    L = hip.lib()
+    rng = np.random.default_rng(tokens * 31 + heads)
+    shape = (tokens, heads, 128)
+    q, k, v = (rng.standard_normal(shape, dtype=np.float32) * 0.5 for _ in range(3))
+    if valid is not None:
+        k[valid:] *= 30.0  # a dropped limit would let these keys dominate
+    cfg = host.Config(tokens, heads, heads, 128) if valid is None else host.Config(tokens, heads, heads, 128, valid=valid)
+    d0 = L.zdraw_hip_dispatch_count()
+    got = ctx.run(q, k, v, cfg)
+    assert L.zdraw_hip_dispatch_count() - d0 == 2  # the rounding launch and the attention launch
+    want = zo.attention_run(q, k, v, oracle_cfg(cfg))
+    mx, mean = refimpl.check_close(got, want, f"long plain {tokens}x{heads} valid={valid}")
+    assert mx <= 4e-3
+    assert np.array_equal(got.view(np.uint32), ctx.run(q, k, v, cfg).view(np.uint32))
+
+
 @pytest.mark.parametrize("tokens,heads,dim,kv,causal", [
     (1, 2, 8, 2, False), (31, 2, 16, 1, False), (97, 3, 64, 3, True), (16, 1, 256, 1, False),
     (40, 4, 128, 2, False), (40, 2, 128, 2, True),

@@ -166,6 +166,8 @@ bool need(const void* handle, size_t bytes) {
     return b && b->ptr && b->len >= bytes && ((uintptr_t)b->ptr % 16) == 0;
 }
 
+constexpr uint32_t kRoundPlainTokens = 1024; // plain f32 attention from this length on rounds its operands once, ahead of the kernel
+
 struct FusedPlan {
     AttnArgs args;
     int in_dtype;
@@ -414,6 +416,48 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
             plan->args.v_bs = pr.y_bs; plan->args.v_ts = pr.y_ts; plan->args.v_hs = pr.y_hs;
             plan->in_dtype = kBF16;
         }
+    }
+    if (x->qk_mode == ZDRAW_HIP_QK_NONE && x->in_dtype == ZDRAW_HIP_F32 && p->tokens >= kRoundPlainTokens) {
+        // Plain attention on f32 rows (the reference's base entry, metal_c.zig:286-299, takes
+        // them): Q (with the softmax scale), K and V are rounded to bf16 once, head-major, into
+        // slots 0-2 by one launch, and the kernel is the direct-to-LDS build, as for prepared
+        // operands. Short sequences stay on the build that rounds in its tile load.
+        const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * 2;
+        Buffer* sc[3];
+        for (int i = 0; i < 3; i++) {
+            sc[i] = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, i, bytes));
+            if (!sc[i]) {
+                set_err("scratch allocation failed");
+                return ZDRAW_HIP_ERR_HANDLE;
+            }
+        }
+        PrepArgs pr;
+        memset(&pr, 0, sizeof(pr));
+        pr.y_bs = (int64_t)p->heads * p->tokens * kHeadDim;
+        pr.y_ts = kHeadDim;
+        pr.y_hs = (int64_t)p->tokens * kHeadDim;
+        pr.tokens = a.tokens; pr.heads = a.heads; pr.batch = a.batch;
+        pr.mode = kQkNone;
+        pr.out_dtype = kBF16;
+        pr.scale = 1.0f;
+        PrepArgs pq = pr, pk = pr, pv = pr;
+        pq.x = a.q; pq.y = sc[0]->ptr; pq.x_bs = a.q_bs; pq.x_ts = a.q_ts; pq.x_hs = a.q_hs; pq.scale = a.scale_log2;
+        pk.x = a.k; pk.y = sc[1]->ptr; pk.x_bs = a.k_bs; pk.x_ts = a.k_ts; pk.x_hs = a.k_hs;
+        pv.x = a.v; pv.y = sc[2]->ptr; pv.x_bs = a.v_bs; pv.x_ts = a.v_ts; pv.x_hs = a.v_hs;
+        plan->prep_q = pq;
+        plan->prep = pk;
+        plan->prep_v = pv;
+        plan->round_v = true;
+        plan->prepass = true;
+        plan->prep_in_dtype = kF32;
+        plan->in_dtype = kBF16;
+        plan->args.q = sc[0]->ptr;
+        plan->args.k = sc[1]->ptr;
+        plan->args.v = sc[2]->ptr;
+        plan->args.q_bs = plan->args.k_bs = plan->args.v_bs = pr.y_bs;
+        plan->args.q_ts = plan->args.k_ts = plan->args.v_ts = pr.y_ts;
+        plan->args.q_hs = plan->args.k_hs = plan->args.v_hs = pr.y_hs;
+        plan->args.scale_log2 = 1.0f;
     }
     return ZDRAW_HIP_OK;
 }

@@ -50,6 +50,8 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
             const int head = h0 + 4 * g;
             float x[8];
             unpack8(raw[g], x);
+#pragma unroll
+            for (int i = 0; i < 8; i++) x[i] *= p.scale; // 1, or the softmax scale on un-normalised query rows
             if (tok_ok && head < p.heads) {
                 const int64_t off = (int64_t)seg * p.y_bs + (int64_t)tok * p.y_ts + (int64_t)head * p.y_hs + d0;
                 if (p.out_dtype == kF32) {
@@ -143,9 +145,11 @@ hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipSt
     if (count < 1 || count > 3) return hipErrorInvalidValue;
     const PrepArgs& p = ops[0];
     if (p.batch <= 0 || p.heads <= 0 || p.tokens <= 0 || p.batch * count > 65535) return hipErrorInvalidValue;
+    // all operands round-only (plain attention on f32 rows), or Q and K prepared and a third round-only
+    const bool plain = p.mode == kQkNone;
     for (int i = 1; i < count; i++) {
         if (ops[i].batch != p.batch || ops[i].heads != p.heads || ops[i].tokens != p.tokens) return hipErrorInvalidValue;
-        if (ops[i].mode != (i == 2 ? (int32_t)kQkNone : p.mode)) return hipErrorInvalidValue;
+        if (ops[i].mode != ((i == 2 || plain) ? (int32_t)kQkNone : p.mode)) return hipErrorInvalidValue;
     }
     PrepPair pair;
     for (int i = 0; i < 3; i++) pair.op[i] = ops[i < count ? i : count - 1];
@@ -156,7 +160,7 @@ hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipSt
     const dim3 grid((unsigned)((p.tokens + kPrepTokens - 1) / kPrepTokens), (unsigned)((p.heads + per_pass - 1) / per_pass),
                     (unsigned)(p.batch * count));
     const dim3 block(kPrepTokens * 64);
-    const bool klein = p.mode == kQkKlein;
+    const bool klein = p.mode == kQkKlein || plain; // round-only operands never reach the mode's code
     if (!klein && p.mode != kQkZimage) return hipErrorInvalidValue;
 #define ZD_PREP(T, M) \
     do { \
