@@ -611,27 +611,46 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
     store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, l32, h);
 }
 
-// Adds the parts of the k-split tiles in part order and writes C. One thread per 16 bytes of
-// a partial tile: thread (tile, wave, e = 16 i + 4 j + r, lane) owns row
-// 128 (wave / 2) + 32 i + lane % 32 and columns 128 (wave % 2) + 32 j + 8 r + 4 (lane / 32) .. + 4
-// of the tile, as in the four-wave build. Every part's load is sent before the first is used.
+// Adds the parts of the k-split tiles in part order and writes C. A workgroup takes the 32 x
+// 128 block (tile, wave, i) of the four-wave build's accumulation layout: its wave j owns the
+// tiles (i, j), a lane row 32 i + lane % 32 and, for r < 4, columns 32 j + 8 r + 4 (lane / 32)
+// .. + 4. Every part's load (4 x splits of 16 bytes per lane) is sent before the first is
+// used; the sums are turned through LDS so that C is stored as whole rows of the block.
 constexpr int kMaxKSplits = 8;
-template <bool F16>
-__global__ void __launch_bounds__(256) gemm_merge_kernel(const GemmArgs g, int c_is_f32) {
-    const int t = (int)blockIdx.x >> 6;
-    const int idx = (((int)blockIdx.x & 63) << 8) + (int)threadIdx.x;
-    const int wave = idx >> 12, e = (idx >> 6) & 63, lane = idx & 63;
-    const f32x4* src = reinterpret_cast<const f32x4*>(g.part) + ((((int64_t)t * g.splits) * 4 + wave) * 64 + e) * 64 + lane;
-    f32x4 v[kMaxKSplits];
+template <bool F16, typename TC>
+__global__ void __launch_bounds__(256) gemm_merge_kernel(const GemmArgs g) {
+    constexpr int ES = (int)sizeof(TC);
+    constexpr int PITCH = 128 * ES + 16; // bytes per staged row
+    __shared__ __attribute__((aligned(16))) unsigned char stage[32 * PITCH];
+    const int t = (int)blockIdx.x >> 4;
+    const int wave = ((int)blockIdx.x >> 2) & 3, i = (int)blockIdx.x & 3;
+    const int j = (int)threadIdx.x >> 6, lane = (int)threadIdx.x & 63;
+    const f32x4* src = reinterpret_cast<const f32x4*>(g.part) +
+                       ((((int64_t)t * g.splits) * 4 + wave) * 64 + (16 * i + 4 * j)) * 64 + lane;
+    f32x4 v[kMaxKSplits][4];
 #pragma unroll
-    for (int z = 0; z < kMaxKSplits; z++) {
-        v[z] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (z < g.splits) v[z] = src[(int64_t)z * (4 * 64 * 64)];
+    for (int z = 0; z < kMaxKSplits; z++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            v[z][r] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (z < g.splits) v[z][r] = src[(int64_t)z * (4 * 64 * 64) + r * 64];
+        }
+    const int l32 = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        f32x4 sum = v[0][r];
+#pragma unroll
+        for (int z = 1; z < kMaxKSplits; z++)
+            if (z < g.splits) sum += v[z][r];
+        unsigned char* dst = stage + l32 * PITCH + (32 * j + 8 * r + 4 * h) * ES;
+        if constexpr (ES == 4) {
+            *reinterpret_cast<f32x4*>(dst) = sum;
+        } else {
+            if constexpr (F16) *reinterpret_cast<u32x2*>(dst) = __builtin_bit_cast(u32x2, __builtin_convertvector(sum, f16x4));
+            else *reinterpret_cast<u32x2*>(dst) = __builtin_bit_cast(u32x2, __builtin_convertvector(sum, bf16x4));
+        }
     }
-    f32x4 sum = v[0];
-#pragma unroll
-    for (int z = 1; z < kMaxKSplits; z++)
-        if (z < g.splits) sum += v[z];
+    __syncthreads();
 
     const int tiles_row = g.tiles_n * g.groups;
     int tm, tn;
@@ -639,30 +658,28 @@ __global__ void __launch_bounds__(256) gemm_merge_kernel(const GemmArgs g, int c
     const int grp = tn / g.tiles_n;
     tn -= grp * g.tiles_n;
     void* const cp = grp == 0 ? g.c : g.c_more[grp - 1];
-    const int i = e >> 4, j = (e >> 2) & 3, r = e & 3;
-    const int row = tm * BM + (wave >> 1) * 128 + 32 * i + (lane & 31);
-    const int col = tn * BN + (wave & 1) * 128 + 32 * j + 8 * r + 4 * (lane >> 5);
-    if (row >= g.m) return;
-    if (c_is_f32) {
-        float* dst = reinterpret_cast<float*>(cp) + (int64_t)row * g.ldc + col;
-        if (col + 3 < g.n && g.ldc % 4 == 0 && reinterpret_cast<uintptr_t>(cp) % 16 == 0) {
-            *reinterpret_cast<f32x4*>(dst) = sum;
+    const int row0 = tm * BM + (wave >> 1) * 128 + 32 * i;
+    const int col0 = tn * BN + (wave & 1) * 128;
+    constexpr int PER = 16 / ES;       // elements per 16-byte chunk
+    constexpr int CH = 128 / PER;      // chunks per row of the block
+    const bool vec = (g.ldc % PER == 0) && (reinterpret_cast<uintptr_t>(cp) % 16 == 0);
+#pragma unroll
+    for (int q = 0; q < 32 * CH / 256; q++) {
+        const int c = (int)threadIdx.x + 256 * q;
+        const int rr = c / CH, cc = c % CH;
+        const int row = row0 + rr, col = col0 + PER * cc;
+        if (row >= g.m || col >= g.n) continue;
+        const u32x4 x = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + cc * 16);
+        TC* dst = reinterpret_cast<TC*>(cp) + (int64_t)row * g.ldc + col;
+        if (vec && col + PER <= g.n) {
+            *reinterpret_cast<u32x4*>(dst) = x;
         } else {
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++)
-                if (col + jj < g.n) dst[jj] = sum[jj];
-        }
-    } else {
-        u32x2 pk;
-        if constexpr (F16) pk = __builtin_bit_cast(u32x2, __builtin_convertvector(sum, f16x4));
-        else pk = __builtin_bit_cast(u32x2, __builtin_convertvector(sum, bf16x4));
-        unsigned short* dst = reinterpret_cast<unsigned short*>(cp) + (int64_t)row * g.ldc + col;
-        if (col + 3 < g.n && g.ldc % 4 == 0 && reinterpret_cast<uintptr_t>(cp) % 8 == 0) {
-            *reinterpret_cast<u32x2*>(dst) = pk;
-        } else {
-#pragma unroll
-            for (int jj = 0; jj < 4; jj++)
-                if (col + jj < g.n) dst[jj] = (unsigned short)(pk[jj >> 1] >> (16 * (jj & 1)));
+            for (int e = 0; e < PER; e++) {
+                if (col + e >= g.n) break;
+                if constexpr (ES == 4) reinterpret_cast<unsigned*>(dst)[e] = x[e];
+                else reinterpret_cast<unsigned short*>(dst)[e] = (unsigned short)(x[e >> 1] >> (16 * (e & 1)));
+            }
         }
     }
 }
@@ -743,7 +760,7 @@ static hipError_t launch_one(const GemmArgs& g0, hipStream_t stream) {
                 gemm_ring_kernel<F16, TC><<<dim3((unsigned)(tail * g0.splits)), dim3(256), kRingLdsBytes, stream>>>(g);
                 hipError_t e = hipGetLastError();
                 if (e != hipSuccess) return e;
-                gemm_merge_kernel<F16><<<dim3((unsigned)tail * 64u), dim3(256), 0, stream>>>(g, std::is_same<TC, float>::value ? 1 : 0);
+                gemm_merge_kernel<F16, TC><<<dim3((unsigned)tail * 16u), dim3(256), 0, stream>>>(g);
             }
             return hipGetLastError();
         }
