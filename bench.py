@@ -369,12 +369,17 @@ def main():
     ap.add_argument("--dynamic-max", action="store_true", help="withhold the score bound (running-maximum softmax)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only sustained-rate probe")
+    ap.add_argument("--cu-count", type=int, default=0,
+                    help="confine the library's stream to this many compute units (0 = all): shows whether "
+                         "the kernel's time follows the CU count or the board's power limit")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a known-size kernel to scale "
                          "the profiler's FETCH_SIZE / WRITE_SIZE counters against)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)")
+    if args.cu_count > 0:
+        os.environ["ZDRAW_HIP_CU_COUNT"] = str(args.cu_count)  # read when the library creates its stream
     if args.path == "gemm":
         return gemm_main(args)
     if args.path == "chain":
@@ -468,6 +473,7 @@ def main():
             "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
             f"tflops_with_k_site_{other}": flops / (o_wall / 100) / 1e12,
             "untimed_spinup_launches": spun,
+            **({"cu_count": args.cu_count} if args.cu_count > 0 else {}),
         },
         "roofline": {
             "bound": "mfma",

@@ -124,7 +124,9 @@ typedef struct ZdrawHipQkOperands {
  * (the caller's error.MetalNotAvailable). */
 void* zdraw_hip_create_device(void);
 void zdraw_hip_release_device(void* device);
-void* zdraw_hip_create_queue(void* device); /* one HIP stream, default priority */
+/* One HIP stream, default priority. Measurement aid: with ZDRAW_HIP_CU_COUNT=n in the
+ * environment (0 < n < the device's CU count) the stream is confined to n compute units. */
+void* zdraw_hip_create_queue(void* device);
 void zdraw_hip_release_queue(void* queue);
 
 /* ---- buffers (metal_c.zig:12-33) ----------------------------------------- */

@@ -777,6 +777,20 @@ void* zdraw_hip_create_queue(void* device) {
     Device* d = static_cast<Device*>(device);
     if (!d) return nullptr;
     hipStream_t s;
+    // Measurement aid: ZDRAW_HIP_CU_COUNT = n confines the stream to n compute units (mask bit
+    // i set for i < n; the driver deals the bits out over the XCDs in turn). It answers "does
+    // the kernel's time depend on how many CUs it has, or on the board's power limit".
+    const char* cus = getenv("ZDRAW_HIP_CU_COUNT");
+    const int ncu = cus ? atoi(cus) : 0;
+    if (ncu > 0 && ncu < d->cus) {
+        std::vector<uint32_t> mask((size_t)(d->cus + 31) / 32, 0u);
+        for (int i = 0; i < ncu; i++) mask[(size_t)i >> 5] |= 1u << (i & 31);
+        if (hipExtStreamCreateWithCUMask(&s, (uint32_t)mask.size(), mask.data()) != hipSuccess) {
+            set_err("hipExtStreamCreateWithCUMask failed");
+            return nullptr;
+        }
+        return new Queue{d, s};
+    }
     if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) {
         set_err("hipStreamCreate failed");
         return nullptr;
