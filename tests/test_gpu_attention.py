@@ -465,6 +465,24 @@ def test_clock_probe_reports_every_workgroup_and_leaves_results_alone(ctx):
     res.release()
 
 
+def test_queue_confined_to_fewer_compute_units_gives_the_same_bits(ctx, monkeypatch):
+    # ZDRAW_HIP_CU_COUNT (a measurement aid) only changes where workgroups run
+    w = wl.by_name("klein_1024", seed=4, small=True)
+    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_PREPASS)
+    base = res.run()
+    res.release()
+    monkeypatch.setenv("ZDRAW_HIP_CU_COUNT", "64")
+    masked = host.Context.init()
+    monkeypatch.delenv("ZDRAW_HIP_CU_COUNT")
+    try:
+        res = wl.Resident(masked, w, dtype=hip.BF16, k_site=hip.K_PREPASS)
+        got = res.run()
+        res.release()
+    finally:
+        masked.deinit()
+    assert np.array_equal(base.view(np.uint32), got.view(np.uint32))
+
+
 def test_scratch_is_grow_only_and_filled(ctx):
     # metal_api.m:6147-6191: a slot is (re)allocated only to grow, and a new allocation is
     # filled before anyone reads it. The library uses the slots itself (pre-passed Q and K,
