@@ -577,12 +577,12 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
             for (int j = 0; j < 16; j++) s_next[qi][j] = 0.f;
 
-        float t[QB][7], mc[QB], alpha[QB], psum[QB];
+        float mc[QB], alpha[QB], psum[QB];
         unsigned pc[QB][8] = {}; // P as packed bf16 pairs
-        bool grew = false;
 #pragma unroll
         for (int qi = 0; qi < QB; qi++) {
-            mc[qi] = 0.f;
+            // watched build: the exponentials are taken against the reference point as it stands
+            mc[qi] = (!BOUNDED && m_run[qi] != -INFINITY) ? m_run[qi] : 0.f;
             alpha[qi] = 1.f;
             psum[qi] = 0.f;
         }
@@ -615,38 +615,9 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                         pin(l_run[qi]);
                     }
                 } else {
-                    if (c == 0) {
-                        t[qi][0] = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
-                        t[qi][1] = fmaxf(fmaxf(sv[3], sv[4]), sv[5]);
-                        t[qi][2] = fmaxf(fmaxf(sv[6], sv[7]), sv[8]);
-                        t[qi][3] = fmaxf(fmaxf(sv[9], sv[10]), sv[11]);
-                    } else if (c == 1) {
-                        t[qi][4] = fmaxf(fmaxf(sv[12], sv[13]), sv[14]);
-                        t[qi][5] = fmaxf(fmaxf(t[qi][0], t[qi][1]), t[qi][2]);
-                        t[qi][6] = fmaxf(fmaxf(t[qi][3], t[qi][4]), sv[15]);
-                        t[qi][0] = fmaxf(t[qi][5], t[qi][6]);
-                    } else if (c == 2) {
-                        // Lazy running maximum (exp2 domain): the reference point of the
-                        // exponentials only moves when this block's maximum exceeds it by
-                        // more than kTau, so P stays within [0, 2^kTau] and O is rescaled on
-                        // a handful of blocks instead of on every new row maximum.
-                        const float mlc = pair_max(t[qi][0]);
-                        const bool up = mlc > m_run[qi] + kTau;
-                        const float m_new = up ? mlc : m_run[qi];
-                        mc[qi] = (m_new == -INFINITY) ? 0.f : m_new;
-                        alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - mc[qi]);
-                        grew |= up;
-                        m_run[qi] = m_new;
-                        pin(mc[qi]);
-                        pin(alpha[qi]);
-                    } else if (c <= 14) {
-                        // pairs on slices 3,4, 6,7, 9,10, 12,13
-                        const int r = c - 3;
-                        if (r % 3 != 2) exp_pair(qi, (r / 3) * 2 + (r % 3));
-                    } else {
-                        l_run[qi] = l_run[qi] * alpha[qi] + psum[qi];
-                        pin(l_run[qi]);
-                    }
+                    // running-maximum build: the same slices, taken against the reference point
+                    // as it stands; the watch after the slots adds the denominator
+                    if ((c & 1) == 0) exp_pair(qi, c >> 1);
                 }
                 if (c == 15) {
                     p_cur[qi][0] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][0], pc[qi][1], pc[qi][2], pc[qi][3]});
@@ -688,14 +659,53 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        // O is relative to m(b-1) here; move it to m(b) before block b's update lands
-        if (!BOUNDED && __any(grew)) {
+        if constexpr (!BOUNDED) {
+            // Lazy running maximum without a maximum per block. The exponentials above were
+            // taken against the reference point m_run as it stood. A lane's 16 of them add up
+            // to more than 16 * 2^kTau only if one of its scores lies more than kTau above the
+            // reference (then, or for a row that has no reference yet, or when the sum is not a
+            // number, the block is redone below); otherwise every P is at most 2^(kTau+4) and
+            // the block stands. The redo forms the row maxima, moves the reference of the rows
+            // whose maximum exceeds it by more than kTau (both lanes of a row decide alike),
+            // takes the exponentials again and rescales O and the denominator.
+            bool redo = false;
 #pragma unroll
-            for (int qi = 0; qi < QB; qi++)
+            for (int qi = 0; qi < QB; qi++) redo |= !(psum[qi] <= 16.0f * 256.0f) || m_run[qi] == -INFINITY;
+            static_assert(kTau == 8.0f, "the watch threshold is 16 * 2^kTau");
+            if (__any(redo)) {
 #pragma unroll
-                for (int blk = 0; blk < 4; blk++)
+                for (int qi = 0; qi < QB; qi++) {
+                    f32x16& sv = s_cur[qi];
+                    float t0 = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
+                    float t1 = fmaxf(fmaxf(sv[3], sv[4]), sv[5]);
+                    float t2 = fmaxf(fmaxf(sv[6], sv[7]), sv[8]);
+                    float t3 = fmaxf(fmaxf(sv[9], sv[10]), sv[11]);
+                    float t4 = fmaxf(fmaxf(sv[12], sv[13]), sv[14]);
+                    t0 = fmaxf(fmaxf(t0, t1), t2);
+                    t3 = fmaxf(fmaxf(t3, t4), sv[15]);
+                    const float mlc = pair_max(fmaxf(t0, t3));
+                    const bool up = mlc > m_run[qi] + kTau;
+                    const float m_new = up ? mlc : m_run[qi];
+                    mc[qi] = (m_new == -INFINITY) ? 0.f : m_new;
+                    alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - mc[qi]);
+                    m_run[qi] = m_new;
+                    psum[qi] = 0.f;
 #pragma unroll
-                    for (int j = 0; j < 16; j++) oacc[qi][blk][j] *= alpha[qi];
+                    for (int pr = 0; pr < 8; pr++) exp_pair(qi, pr);
+                    l_run[qi] *= alpha[qi];
+#pragma unroll
+                    for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                        for (int j = 0; j < 16; j++) oacc[qi][blk][j] *= alpha[qi];
+                    p_cur[qi][0] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][0], pc[qi][1], pc[qi][2], pc[qi][3]});
+                    p_cur[qi][1] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][4], pc[qi][5], pc[qi][6], pc[qi][7]});
+                }
+            }
+#pragma unroll
+            for (int qi = 0; qi < QB; qi++) {
+                l_run[qi] += psum[qi];
+                pin(l_run[qi]);
+            }
         }
         if (sync) {
             if constexpr (XSTEP) {
