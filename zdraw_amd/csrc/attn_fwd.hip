@@ -109,8 +109,10 @@ __device__ __forceinline__ void pin(T& v) {
 // BOUNDED: the caller has promised that every scaled score fits comfortably in
 // the fp32 exponent (QK-normalised operands: |q'.k'|/sqrt(D) <= sqrt(D) max|w_q| max|w_k|).
 // Softmax is shift-invariant, so the kernel then exponentiates the scores as
-// they are: no running maximum, no subtraction, no rescale of O. Otherwise the
-// lazy running maximum below is used.
+// they are: no running maximum, no subtraction, no rescale of O. Otherwise a
+// lazy running maximum is kept: S accumulates on top of minus the reference point
+// (the MFMA's C operand), so the exponentials need no subtraction either, and the
+// block's row sums, not a maximum per block, say when the reference must move.
 template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
 __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(const AttnArgs a) {
     constexpr int NT = NW * 64;
@@ -428,6 +430,18 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         m_run[qi] = -INFINITY;
         l_run[qi] = 0.f;
     }
+    // Running-maximum build: minus the reference point of each query column, in the shape of an
+    // MFMA accumulator. The first MFMA of a block's S takes it as its C operand, so scores arrive
+    // relative to the reference and the exponentials need no subtraction.
+    // (Only the builds with registers to spare: prepared 16-bit operands. The others subtract.)
+    constexpr bool REFACC = !BOUNDED && KMODE == kQkNone && std::is_same<TIn, bf16_t>::value && NW == 8 && QB == 1;
+    f32x16 negm[REFACC ? QB : 1];
+    if constexpr (REFACC) {
+#pragma unroll
+        for (int qi = 0; qi < QB; qi++)
+#pragma unroll
+            for (int j = 0; j < 16; j++) negm[qi][j] = 0.f;
+    }
 
     // LDS byte addresses of this lane's fragments in ring stage 0; a stage, a key half (kb)
     // and a row half add constants. K: key row l32, dims 16 s + 8 h .. +7 (8 addresses, the
@@ -575,22 +589,23 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
         for (int qi = 0; qi < QB; qi++)
 #pragma unroll
-            for (int j = 0; j < 16; j++) s_next[qi][j] = 0.f;
+            for (int j = 0; j < 16; j++) s_next[qi][j] = REFACC ? negm[qi][j] : 0.f;
 
         float mc[QB], alpha[QB], psum[QB];
         unsigned pc[QB][8] = {}; // P as packed bf16 pairs
 #pragma unroll
         for (int qi = 0; qi < QB; qi++) {
-            // watched build: the exponentials are taken against the reference point as it stands
-            mc[qi] = (!BOUNDED && m_run[qi] != -INFINITY) ? m_run[qi] : 0.f;
+            mc[qi] = (!BOUNDED && !REFACC && m_run[qi] != -INFINITY) ? m_run[qi] : 0.f;
             alpha[qi] = 1.f;
             psum[qi] = 0.f;
         }
         // exponentials of elements 2*pr, 2*pr+1 of this lane's 16 scores
-        auto exp_pair = [&](int qi, int pr) __attribute__((always_inline)) {
+        // (`shifted`: the scores still have mc to lose; not so for bounded scores, nor for scores
+        // that arrived relative to the reference point)
+        auto exp_pair = [&](int qi, int pr, auto shifted) __attribute__((always_inline)) {
             f32x16& sv = s_cur[qi];
             f32x2 pp;
-            if constexpr (BOUNDED) {
+            if constexpr (BOUNDED || !decltype(shifted)::value) {
                 pp[0] = __builtin_amdgcn_exp2f(sv[2 * pr]);
                 pp[1] = __builtin_amdgcn_exp2f(sv[2 * pr + 1]);
             } else {
@@ -609,15 +624,16 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             for (int qi = 0; qi < QB; qi++) {
                 f32x16& sv = s_cur[qi];
                 if constexpr (BOUNDED) {
-                    if ((c & 1) == 0) exp_pair(qi, c >> 1);
+                    if ((c & 1) == 0) exp_pair(qi, c >> 1, std::false_type{});
                     if (c == 15) {
                         l_run[qi] += psum[qi];
                         pin(l_run[qi]);
                     }
                 } else {
-                    // running-maximum build: the same slices, taken against the reference point
-                    // as it stands; the watch after the slots adds the denominator
-                    if ((c & 1) == 0) exp_pair(qi, c >> 1);
+                    // running-maximum build: the same slices, against the reference point as it
+                    // stands (the scores arrive relative to it, or it is subtracted here); the
+                    // watch after the slots adds the denominator
+                    if ((c & 1) == 0) exp_pair(qi, c >> 1, std::integral_constant<bool, !REFACC>{});
                 }
                 if (c == 15) {
                     p_cur[qi][0] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][0], pc[qi][1], pc[qi][2], pc[qi][3]});
@@ -660,8 +676,9 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         }
 
         if constexpr (!BOUNDED) {
-            // Lazy running maximum without a maximum per block. The exponentials above were
-            // taken against the reference point m_run as it stood. A lane's 16 of them add up
+            // Lazy running maximum without a maximum per block. The exponentials above were taken
+            // against the reference point m_run as it stood (the scores arrived relative to it,
+            // negm being their accumulator's starting value, or it was subtracted). A lane's 16 of them add up
             // to more than 16 * 2^kTau only if one of its scores lies more than kTau above the
             // reference (then, or for a row that has no reference yet, or when the sum is not a
             // number, the block is redone below); otherwise every P is at most 2^(kTau+4) and
@@ -683,15 +700,26 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                     float t4 = fmaxf(fmaxf(sv[12], sv[13]), sv[14]);
                     t0 = fmaxf(fmaxf(t0, t1), t2);
                     t3 = fmaxf(fmaxf(t3, t4), sv[15]);
-                    const float mlc = pair_max(fmaxf(t0, t3));
+                    // the scores are relative to `ref` (the reference point, 0 before the first)
+                    const float ref = (REFACC && m_run[qi] != -INFINITY) ? m_run[qi] : 0.f;
+                    const float mlc = pair_max(fmaxf(t0, t3)) + ref;
                     const bool up = mlc > m_run[qi] + kTau;
                     const float m_new = up ? mlc : m_run[qi];
-                    mc[qi] = (m_new == -INFINITY) ? 0.f : m_new;
-                    alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - mc[qi]);
+                    const float ref_new = (m_new == -INFINITY) ? 0.f : m_new;
+                    mc[qi] = ref_new - ref;
+                    alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - ref_new);
                     m_run[qi] = m_new;
                     psum[qi] = 0.f;
 #pragma unroll
-                    for (int pr = 0; pr < 8; pr++) exp_pair(qi, pr);
+                    for (int pr = 0; pr < 8; pr++) exp_pair(qi, pr, std::true_type{});
+                    if constexpr (REFACC) {
+                        // the next block's scores were formed against the old reference
+#pragma unroll
+                        for (int j = 0; j < 16; j++) {
+                            s_next[qi][j] -= mc[qi];
+                            negm[qi][j] = -ref_new;
+                        }
+                    }
                     l_run[qi] *= alpha[qi];
 #pragma unroll
                     for (int blk = 0; blk < 4; blk++)
