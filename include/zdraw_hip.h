@@ -339,7 +339,10 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
  * measurement), run back to back for about `milliseconds` on the current device;
  * the last launch's TFLOP/s is returned. random_operands != 0 feeds normally
  * distributed operands, 0 feeds constants: the board's power limit makes the
- * first markedly slower, and it is the ceiling that applies to real data. */
+ * first markedly slower, and it is the ceiling that applies to real data.
+ * random_operands 2, 3, 5: normally distributed operands with the B operand held
+ * over 2, 4, 8 consecutive MFMAs; 4: the A operand held over 2 (how much of the
+ * power goes with operands that change from one MFMA to the next). */
 int zdraw_hip_mfma_probe(int random_operands, int milliseconds, double* tflops);
 
 /* HIP events on a queue's stream, for measuring kernels where they run. */

@@ -26,6 +26,8 @@ constexpr int kThreads = 512;  // two waves per SIMD
 constexpr int kBlocks = 256;   // one workgroup per CU
 
 // 8 MFMAs per iteration on four independent accumulators; operands stay in registers.
+// SA / SB = how many consecutive MFMAs take the same A / B operand (1 = each its own).
+template <int SA, int SB>
 __global__ void __launch_bounds__(kThreads) mfma_probe_kernel(const bf16x8* __restrict__ data, float* out, int iters) {
     const int t = threadIdx.x;
     bf16x8 a[8], b[8];
@@ -38,10 +40,10 @@ __global__ void __launch_bounds__(kThreads) mfma_probe_kernel(const bf16x8* __re
     for (int it = 0; it < iters; it++) {
 #pragma unroll
         for (int i = 0; i < 8; i += 4) {
-            o0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[i], o0, 0, 0, 0);
-            o1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i + 1], b[i + 1], o1, 0, 0, 0);
-            o2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i + 2], b[i + 2], o2, 0, 0, 0);
-            o3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i + 3], b[i + 3], o3, 0, 0, 0);
+            o0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i / SA * SA], b[i / SB * SB], o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(i + 1) / SA * SA], b[(i + 1) / SB * SB], o1, 0, 0, 0);
+            o2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(i + 2) / SA * SA], b[(i + 2) / SB * SB], o2, 0, 0, 0);
+            o3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(i + 3) / SA * SA], b[(i + 3) / SB * SB], o3, 0, 0, 0);
         }
         if ((it & 63) == 63) { // keep the accumulators finite
 #pragma unroll
@@ -94,7 +96,14 @@ extern "C" int zdraw_hip_mfma_probe(int random_operands, int milliseconds, doubl
         bool ok = true;
         while (ok && total < (float)milliseconds) { // launches back to back; the last one is quoted
             ok = hipEventRecord(e0, nullptr) == hipSuccess;
-            mfma_probe_kernel<<<kBlocks, kThreads>>>(reinterpret_cast<const bf16x8*>(d), out, iters);
+            const bf16x8* src = reinterpret_cast<const bf16x8*>(d);
+            switch (random_operands) { // 2..5: random operands, one side held over consecutive MFMAs
+            case 2: mfma_probe_kernel<1, 2><<<kBlocks, kThreads>>>(src, out, iters); break;
+            case 3: mfma_probe_kernel<1, 4><<<kBlocks, kThreads>>>(src, out, iters); break;
+            case 4: mfma_probe_kernel<2, 1><<<kBlocks, kThreads>>>(src, out, iters); break;
+            case 5: mfma_probe_kernel<1, 8><<<kBlocks, kThreads>>>(src, out, iters); break;
+            default: mfma_probe_kernel<1, 1><<<kBlocks, kThreads>>>(src, out, iters); break;
+            }
             ok = ok && hipGetLastError() == hipSuccess && hipEventRecord(e1, nullptr) == hipSuccess &&
                  hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&last, e0, e1) == hipSuccess;
             total += last;
