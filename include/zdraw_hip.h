@@ -342,7 +342,8 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
  * first markedly slower, and it is the ceiling that applies to real data.
  * random_operands 2, 3, 5: normally distributed operands with the B operand held
  * over 2, 4, 8 consecutive MFMAs; 4: the A operand held over 2 (how much of the
- * power goes with operands that change from one MFMA to the next). */
+ * power goes with operands that change from one MFMA to the next); 6, 7: each
+ * accumulator takes 2, 8 MFMAs in a row instead of one in rotation. */
 int zdraw_hip_mfma_probe(int random_operands, int milliseconds, double* tflops);
 
 /* HIP events on a queue's stream, for measuring kernels where they run. */

@@ -27,7 +27,9 @@ constexpr int kBlocks = 256;   // one workgroup per CU
 
 // 8 MFMAs per iteration on four independent accumulators; operands stay in registers.
 // SA / SB = how many consecutive MFMAs take the same A / B operand (1 = each its own).
-template <int SA, int SB>
+// RUN = how many consecutive MFMAs accumulate into the same registers (1 = the four
+// accumulators in rotation).
+template <int SA, int SB, int RUN = 1>
 __global__ void __launch_bounds__(kThreads) mfma_probe_kernel(const bf16x8* __restrict__ data, float* out, int iters) {
     const int t = threadIdx.x;
     bf16x8 a[8], b[8];
@@ -38,6 +40,20 @@ __global__ void __launch_bounds__(kThreads) mfma_probe_kernel(const bf16x8* __re
     }
     f32x16 o0 = {}, o1 = {}, o2 = {}, o3 = {};
     for (int it = 0; it < iters; it++) {
+        if constexpr (RUN > 1) {
+            // 32 MFMAs per trip of this form: every accumulator takes RUN in a row
+#pragma unroll
+            for (int r = 0; r < 8 / RUN; r++) {
+#pragma unroll
+                for (int i = 0; i < RUN; i++) o0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(RUN * r + i) & 7], b[(RUN * r + i) & 7], o0, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < RUN; i++) o1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(RUN * r + i + 1) & 7], b[(RUN * r + i + 3) & 7], o1, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < RUN; i++) o2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(RUN * r + i + 2) & 7], b[(RUN * r + i + 5) & 7], o2, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < RUN; i++) o3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(RUN * r + i + 3) & 7], b[(RUN * r + i + 7) & 7], o3, 0, 0, 0);
+            }
+        } else
 #pragma unroll
         for (int i = 0; i < 8; i += 4) {
             o0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i / SA * SA], b[i / SB * SB], o0, 0, 0, 0);
@@ -102,6 +118,8 @@ extern "C" int zdraw_hip_mfma_probe(int random_operands, int milliseconds, doubl
             case 3: mfma_probe_kernel<1, 4><<<kBlocks, kThreads>>>(src, out, iters); break;
             case 4: mfma_probe_kernel<2, 1><<<kBlocks, kThreads>>>(src, out, iters); break;
             case 5: mfma_probe_kernel<1, 8><<<kBlocks, kThreads>>>(src, out, iters); break;
+            case 6: mfma_probe_kernel<1, 1, 2><<<kBlocks, kThreads>>>(src, out, iters / 4); break;
+            case 7: mfma_probe_kernel<1, 1, 8><<<kBlocks, kThreads>>>(src, out, iters / 4); break;
             default: mfma_probe_kernel<1, 1><<<kBlocks, kThreads>>>(src, out, iters); break;
             }
             ok = ok && hipGetLastError() == hipSuccess && hipEventRecord(e1, nullptr) == hipSuccess &&
