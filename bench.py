@@ -278,7 +278,7 @@ def wide_main(args):
     qb, kb, vb = ctx.buffer(q), ctx.buffer(k), ctx.buffer(v)
     ob = ctx.buffer(nbytes=q.nbytes)
     err = C.create_string_buffer(128)
-    pipe = L.zdraw_hip_compile(ctx.device, b"attention_wide_mfma", err, 128)
+    pipe = L.zdraw_hip_compile(ctx.device, None, b"attention_wide_mfma", err, 128)
     if not pipe:
         raise RuntimeError(err.value)
     p = hip.AttnParams(tokens, 1, 1, 512, 0, 0)
@@ -368,7 +368,6 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="kernel shape: 0 = 8 waves, 1 = 4 waves x 2 workgroups")
     ap.add_argument("--dynamic-max", action="store_true", help="withhold the score bound (running-maximum softmax)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only sustained-rate probe")
     ap.add_argument("--cu-count", type=int, default=0,
                     help="confine the library's stream to this many compute units (0 = all): shows whether "
                          "the kernel's time follows the CU count or the board's power limit")
@@ -428,14 +427,6 @@ def main():
     if not np.isfinite(out).all():
         raise RuntimeError("non-finite output")
 
-    # what a loop of nothing but MFMAs sustains on this board, for the roofline's context
-    mfma_only = {}
-    if not args.no_mfma_probe:
-        for label, rnd in (("normal_operands", 1), ("constant_operands", 0)):
-            t = C.c_double(0.0)
-            if L.zdraw_hip_mfma_probe(rnd, 600, C.byref(t)) == 0:
-                mfma_only[label] = t.value
-
     # the other K site, for the record (short, untimed by the driver's clock)
     other = "tile" if args.k_site == "prepass" else "prepass"
     res.ext.k_site = hip.K_IN_TILE_LOAD if other == "tile" else hip.K_PREPASS
@@ -485,7 +476,6 @@ def main():
             "kernel": "attn_fwd_kernel",
             "kernel_ms": kern_ms,
             "shader_clock": clock,
-            "mfma_only_sustained_tflops": mfma_only or None,
         },
     }
     res.release()

@@ -101,7 +101,12 @@ typedef struct ZdrawHipAttnExt {
      * rotations it is sqrt(head_dim) * max|w_q| * max|w_k|. A bound of at most 44
      * lets the kernel exponentiate scores without tracking a running maximum
      * (softmax is shift-invariant); 0 or a larger bound selects the running-maximum
-     * form. A bound that is too small is a caller error (overflow). */
+     * form. When the call carries norm weights (qk_mode != NONE) the library forms
+     * sqrt(head_dim) * max|w_q| * max|w_k| from the weight buffers itself (read once
+     * per buffer, until the buffer is written or released) and decides on the larger of
+     * the two values: the caller's figure can only make the choice more cautious, a figure
+     * that is too small cannot overflow. With qk_mode NONE there are no weights to check
+     * and the caller's figure stands. */
     float score_bound;
     uint32_t reserved;
 } ZdrawHipAttnExt;
@@ -124,8 +129,7 @@ typedef struct ZdrawHipQkOperands {
  * (the caller's error.MetalNotAvailable). */
 void* zdraw_hip_create_device(void);
 void zdraw_hip_release_device(void* device);
-/* One HIP stream, default priority. Measurement aid: with ZDRAW_HIP_CU_COUNT=n in the
- * environment (0 < n < the device's CU count) the stream is confined to n compute units. */
+/* One HIP stream, default priority. */
 void* zdraw_hip_create_queue(void* device);
 void zdraw_hip_release_queue(void* queue);
 
@@ -143,10 +147,11 @@ void* zdraw_hip_buffer_device_ptr(void* buffer); /* no reference counterpart: in
 void zdraw_hip_release_buffer(void* buffer);
 
 /* ---- pipelines (metal_c.zig:99-107) -------------------------------------- */
-/* The kernels are compiled ahead of time for gfx950, so "compile" is a lookup
- * by entry name: "attention_block_mfma" (the only attention pipeline),
+/* Same argument list as zdraw_metal_compile (metal_c.zig:99-105). The kernels are
+ * compiled ahead of time for gfx950, so `source` is not read (NULL is accepted) and
+ * "compile" is a lookup by entry name: "attention_block_mfma", "attention_wide_mfma",
  * "qk_norm_rope" and "gemm_half". Unknown names return NULL and write a message. */
-void* zdraw_hip_compile(void* device, const char* entry, char* error_buf, size_t error_len);
+void* zdraw_hip_compile(void* device, const char* source, const char* entry, char* error_buf, size_t error_len);
 void zdraw_hip_release_pipeline(void* pipeline);
 size_t zdraw_hip_pipeline_threads(void* pipeline);
 
@@ -179,12 +184,34 @@ int zdraw_hip_run_attention_fused(void* queue, void* q, void* k, void* v, void* 
                                   const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
                                   const ZdrawHipQkOperands* ops);
 
-/* ---- standalone QK-norm + rope (metal_c.zig:148-159, QkNormParams :258-274) -
- * In place on f32 token-major q [tokens][heads][128] and k [tokens][kv_heads][128].
- * Only ext->qk_mode, eps, txt_rows, zimage_* and rope_batch_rows are read. */
-int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
-                               const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
-                               const ZdrawHipQkOperands* ops);
+/* ---- standalone QK-norm + rope --------------------------------------------
+ * The general form (no counterpart declaration in the reference; it also serves the
+ * in-place Klein krms_rope dispatches, klein/zflux2_resident.zig:1573-1579). In place on
+ * f32 token-major q [tokens][heads][128] and k [tokens][kv_heads][128]. Only
+ * ext->qk_mode, eps, txt_rows, zimage_* and rope_batch_rows are read. Blocks until done. */
+int zdraw_hip_run_qk_norm_rope_ext(void* queue, void* pipeline, void* q, void* k,
+                                   const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                                   const ZdrawHipQkOperands* ops);
+
+/* metal_c.zig:148-159 with QkNormParams (metal_c.zig:258-274), argument for argument: the
+ * Z-Image qk_norm_rope dispatch behind mqk.run (metal/mqk.zig:20-58). In place on f32
+ * token-major q [tokens][heads][head_dim] and k [tokens][kv_heads][head_dim]; q_weight /
+ * k_weight hold head_dim norm weights of type params->q_dtype / k_dtype at byte offsets
+ * params->q_offset / k_offset; pos is u64 [tokens][3]; rope the (cos,sin) f32 pair table
+ * (zrope.Cache.pairBytes) whose axes start at params->base0..2 pairs. thread_count is
+ * accepted and not used. A position past its axis (zimage/zrope.zig:48 refuses those on the
+ * host) reads the axis's last table entry instead of memory outside the table. Blocks until
+ * done; returns 0, or 1 / 2 / negative as above. */
+typedef struct ZdrawQkNormParams { /* metal_c.zig:258-274, 80 bytes */
+    uint32_t tokens, heads, kv_heads, head_dim;
+    uint32_t q_dtype, k_dtype; /* element type of q_norm / k_norm: 1 f16, 2 bf16, 3 f32 */
+    uint32_t dim0, dim1, dim2; /* rope axis widths, sum = head_dim */
+    float eps;
+    uint64_t q_offset, k_offset; /* byte offsets of the norm weights in their buffers */
+    uint64_t base0, base1, base2; /* axis bases in (cos,sin) pairs */
+} ZdrawQkNormParams;
+int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k, void* q_weight, void* k_weight,
+                               void* pos, void* rope, const ZdrawQkNormParams* params, size_t thread_count);
 
 /* ---- projections either side of attention: C = A x W^T ----------------------
  * metal_c.zig:276-283 (GemmParams), same field order, 32 bytes. dtype is the
@@ -259,14 +286,6 @@ int zdraw_hip_run_gemm_group_ext_enc(void* batch, void* a, void* const* ws, void
  * ZdrawBlockChainParams (metal_api.m:5961-5987) that this segment reads, in the
  * reference's order. Rows padded to a multiple of 32 (zimage/zseq.zig:23-34) are
  * ordinary rows here, as they are there. */
-typedef struct ZdrawQkNormParams { /* metal_c.zig:258-274, 80 bytes */
-    uint32_t tokens, heads, kv_heads, head_dim;
-    uint32_t q_dtype, k_dtype; /* element type of q_norm / k_norm: 1 f16, 2 bf16, 3 f32 */
-    uint32_t dim0, dim1, dim2; /* rope axis widths, sum = head_dim */
-    float eps;
-    uint64_t q_offset, k_offset; /* byte offsets of the norm weights in their buffers */
-    uint64_t base0, base1, base2; /* axis bases in (cos,sin) pairs */
-} ZdrawQkNormParams;
 
 typedef struct ZdrawHipChainAttnBuffers {
     void* norm; /* [tokens][hidden] layer input after its norm (activation dtype) */
@@ -326,26 +345,6 @@ uint64_t zdraw_hip_gpu_ns(void); /* device time summed over completed batches / 
 void zdraw_hip_trace_attention(int on);
 uint64_t zdraw_hip_trace_attention_ns(uint64_t* launches);
 
-/* Clock probe (no reference counterpart: measurement). While on, every workgroup
- * of an attention launch records how long it ran in shader-clock cycles and in
- * ticks of the fixed 100 MHz reference counter; cycles / ticks x 0.1 is the clock
- * in GHz that the kernel really ran at (under load the power limit sets it).
- * clock_probe_read waits for the last probed launch and copies the first
- * `capacity` workgroups' figures (in launch order); it returns how many. */
-void zdraw_hip_clock_probe(int on);
-size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t capacity);
-
-/* Sustained rate of a loop of nothing but bf16 MFMAs (no reference counterpart:
- * measurement), run back to back for about `milliseconds` on the current device;
- * the last launch's TFLOP/s is returned. random_operands != 0 feeds normally
- * distributed operands, 0 feeds constants: the board's power limit makes the
- * first markedly slower, and it is the ceiling that applies to real data.
- * random_operands 2, 3, 5: normally distributed operands with the B operand held
- * over 2, 4, 8 consecutive MFMAs; 4: the A operand held over 2 (how much of the
- * power goes with operands that change from one MFMA to the next); 6, 7: each
- * accumulator takes 2, 8 MFMAs in a row instead of one in rotation. */
-int zdraw_hip_mfma_probe(int random_operands, int milliseconds, double* tflops);
-
 /* HIP events on a queue's stream, for measuring kernels where they run. */
 void* zdraw_hip_event_create(void);
 int zdraw_hip_event_record(void* event, void* queue);
@@ -353,12 +352,6 @@ int zdraw_hip_event_sync(void* event);
 float zdraw_hip_event_elapsed_ms(void* start, void* stop); /* negative on error */
 void zdraw_hip_event_release(void* event);
 int zdraw_hip_queue_sync(void* queue);
-
-/* Measurement knob: which build of the attention kernel runs. Bit 0:
- * 0 = 8 waves x 32 query rows per workgroup, one workgroup per CU (default);
- * 1 = 4 waves x 32 query rows, two workgroups per CU. Bit 1: 2 = never split the
- * tiles of a thinly filled last round along the keys (by default they are). */
-void zdraw_hip_set_attention_variant(int variant);
 
 /* How a launch of `tiles` workgroup tiles (segments x heads x query blocks) is laid on `cus`
  * compute units (no reference counterpart: scheduling, exposed so that it can be checked
@@ -376,9 +369,13 @@ void zdraw_hip_attention_tail_plan(uint64_t tiles, uint32_t cus, uint32_t key_bl
 void zdraw_hip_gemm_tail_plan(uint32_t m, uint32_t k, uint32_t n, uint32_t groups, uint32_t cus, uint32_t* tail_tiles,
                               uint32_t* splits);
 
-/* Measurement knob: which build multiplies 256 x 256 tiles of 16-bit activations.
- * 1 = four waves, 128 x 128 each (default); 0 = eight waves, 64 x 128 each. */
-void zdraw_hip_set_gemm_build(int build);
+/* Positions per Z-Image rope axis that lie inside a (cos,sin) pair table of `table_bytes`
+ * bytes whose axes start at base[0..2] pairs and are dims[0..2] wide (no reference
+ * counterpart: zimage/zrope.zig:48 refuses pos >= len on the host; positions that are only
+ * known on the device are held to these counts by the kernels, so that none indexes outside
+ * the table). For the layout of zrope.Cache the counts are its `lens`. Host arithmetic only.
+ * 0, or 2 when an axis has no whole position inside the table. */
+int zdraw_hip_zimage_axis_lens(uint64_t table_bytes, const uint64_t* base, const uint32_t* dims, uint32_t* lens);
 
 /* ABI drift guard (src/abi_gen.zig, runtime/abi_assert.zig:29): sizeof of the
  * shared structs as this library was compiled. which: 0 = ZdrawAttnParams,

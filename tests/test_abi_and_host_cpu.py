@@ -15,9 +15,16 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def header_symbols():
-    text = open(os.path.join(ROOT, "include", "zdraw_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(zdraw_hip_[a-z0-9_]+)\s*\(", text)))
+    """Every function include/*.h declares (the boundary and the measurement aids)."""
+    names = set()
+    inc = os.path.join(ROOT, "include")
+    headers = sorted(f for f in os.listdir(inc) if f.endswith(".h"))
+    assert "zdraw_hip.h" in headers and "zdraw_hip_measure.h" in headers
+    for h in headers:
+        text = open(os.path.join(inc, h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(zdraw_hip_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol():
@@ -108,10 +115,41 @@ def test_tail_plan_of_the_baseline_shapes():
         assert (t == 0 and s == 1) or (t == tiles % 256 and 2 <= s <= 16 and t * s <= 256 and 144 // s >= 8)
 
 
+def test_zimage_axis_lens_are_the_positions_the_pair_table_holds():
+    # what the kernels hold device-resident positions to (the reference refuses pos >= len
+    # on the host, zimage/zrope.zig:48): for zrope.Cache's layout the counts are its lens
+    L = hip.lib()
+
+    def lens_of(table_pairs, bases, dims):
+        out = (C.c_uint32 * 3)(7, 7, 7)
+        rc = L.zdraw_hip_zimage_axis_lens(table_pairs * 8, (C.c_uint64 * 3)(*bases), (C.c_uint32 * 3)(*dims), out)
+        return rc, tuple(out)
+
+    cfg = zo.RopeConfig(wl.ZIMAGE_DIMS, wl.ZIMAGE_LENS, wl.ZIMAGE_THETA)
+    bases = zo.zrope_axis_bases(cfg)
+    pairs = zo.zrope_fill(cfg).shape[0]
+    assert lens_of(pairs, bases, wl.ZIMAGE_DIMS) == (0, tuple(wl.ZIMAGE_LENS))
+    # the last position of every axis ends inside the table, the one after it does not
+    order = sorted(range(3), key=lambda a: bases[a])
+    for a in range(3):
+        per = wl.ZIMAGE_DIMS[a] // 2
+        nxt = min([bases[b] for b in range(3) if bases[b] > bases[a]] + [pairs])
+        assert bases[a] + wl.ZIMAGE_LENS[a] * per <= nxt < bases[a] + (wl.ZIMAGE_LENS[a] + 1) * per
+    assert order == [0, 1, 2]
+    # small cases by hand: axes of 2, 4, 4 pairs per position
+    assert lens_of(2 * 3 + 4 * 5 + 4 * 2, (0, 6, 26), (4, 8, 8)) == (0, (3, 5, 2))
+    assert lens_of(2 * 3 + 4 * 5 + 4 * 2 + 3, (0, 6, 26), (4, 8, 8)) == (0, (3, 5, 2))   # a partial position does not count
+    assert lens_of(34, (26, 0, 20), (8, 8, 4)) == (0, (2, 5, 3))                          # axes in any order
+    assert lens_of(29, (0, 6, 26), (4, 8, 8))[0] == hip.INVALID                           # last axis has no whole position
+    assert lens_of(26, (0, 6, 26), (4, 8, 8))[0] == hip.INVALID                           # base at the end of the table
+    assert lens_of(40, (0, 6, 26), (4, 0, 8))[0] == hip.INVALID                           # an axis without pairs
+    assert L.zdraw_hip_zimage_axis_lens(64, None, None, None) == hip.ERR_HANDLE
+
+
 def test_pipeline_lookup_without_device_is_null():
     L = hip.lib()
     err = C.create_string_buffer(128)
-    assert not L.zdraw_hip_compile(None, b"attention_block_mfma", err, 128)
+    assert not L.zdraw_hip_compile(None, None, b"attention_block_mfma", err, 128)
 
 
 def _has_gpu():

@@ -580,3 +580,376 @@ def test_key_split_tail_matches_whole_tiles_and_oracle(ctx, tokens, valid, heads
     assert np.abs(split - whole).max() < 2e-3
     for b in bufs:
         b.release()
+
+
+# ------------------------------------ the running maximum's reference point moves late
+def _planted(tokens, heads, plant, seed):
+    """N(0, 0.25) operands in which even query rows lean on a direction u that only the
+    planted keys carry: key j of `plant` scores about strength[j] (natural-log units) above
+    the field for even rows and nothing for odd rows, so inside one wave some rows move
+    their reference point and their neighbours do not."""
+    rng = np.random.default_rng(seed)
+    shape = (tokens, heads, 128)
+    q, k, v = (rng.standard_normal(shape, dtype=np.float32) * np.float32(0.5) for _ in range(3))
+    u = np.full(128, 1.0 / np.sqrt(128.0), np.float32)
+    alpha = 4.0
+    q[0::2] += np.float32(alpha) * u
+    for key, nats in plant:
+        k[key] = np.float32(nats * np.sqrt(128.0) / alpha) * u
+    rb = lambda a: host.bf16_bits_to_f32(host.f32_to_bf16_bits(a))
+    return rb(q), rb(k), rb(v)
+
+
+def _plain_fused(ctx, q, k, v, *, valid=0, in_dtype, key_pad=None, knob=0):
+    """One blocking plain-attention call (operands used as given) with score_bound 0."""
+    L = hip.lib()
+    tokens, heads = q.shape[0], q.shape[1]
+    conv = host.f32_to_bf16_bits if in_dtype == hip.BF16 else (lambda a: np.ascontiguousarray(a, np.float32))
+    bufs = [ctx.buffer(conv(a)) for a in (q, k, v)]
+    o = ctx.buffer(nbytes=q.size * 4)
+    p = hip.AttnParams(tokens, heads, heads, 128, 0, valid)
+    x = hip.AttnExt()
+    for s_ in (x.q_stride, x.k_stride, x.v_stride, x.out_stride):
+        s_[0], s_[1], s_[2] = 0, heads * 128, 128
+    x.batch, x.in_dtype, x.out_dtype, x.qk_mode, x.score_bound = 1, in_dtype, hip.F32, hip.QK_NONE, 0.0
+    ops = hip.QkOperands()
+    pad = None
+    if key_pad is not None:
+        pad = ctx.buffer(np.ascontiguousarray(key_pad, np.uint8))
+        ops.key_pad = pad.handle
+    L.zdraw_hip_set_attention_variant(knob)
+    try:
+        rc = L.zdraw_hip_run_attention_fused(ctx.queue, bufs[0].handle, bufs[1].handle, bufs[2].handle, o.handle,
+                                             C.byref(p), C.byref(x), C.byref(ops))
+    finally:
+        L.zdraw_hip_set_attention_variant(0)
+    assert rc == 0, hip.last_error()
+    out = o.read(np.float32, q.shape)
+    for b in bufs + [o] + ([pad] if pad is not None else []):
+        b.release()
+    return out
+
+
+# first, a middle and the last key block; rising, so that the reference moves at each of them
+PLANT_CASES = [
+    # name, tokens, heads, in_dtype, valid, planted (key, nats), whole tiles only (knob 2)
+    ("bf16 direct-to-LDS", 1024, 2, hip.BF16, 0, [(5, 21.0), (500, 28.0), (1023, 35.0)], 2),
+    ("bf16 direct-to-LDS, last block only", 2048, 1, hip.BF16, 0, [(2047, 33.0)], 2),
+    ("f32 rows rounded in the tile load", 640, 2, hip.F32, 0, [(3, 21.0), (333, 28.0), (639, 35.0)], 2),
+    ("bf16 masked by a key limit", 1100, 2, hip.BF16, 1000, [(7, 21.0), (480, 28.0), (999, 35.0), (1050, 60.0)], 2),
+    ("bf16 ragged last block", 1001, 2, hip.BF16, 0, [(40, 24.0), (1000, 34.0)], 2),
+    ("f32 masked by a key limit", 700, 1, hip.F32, 650, [(600, 30.0), (649, 36.0), (660, 60.0)], 2),
+    ("key-split parts", 1500, 3, hip.BF16, 0, [(30, 21.0), (820, 28.0), (1310, 35.0)], 0),
+    ("key-split parts, masked", 1500, 3, hip.BF16, 1400, [(700, 25.0), (1399, 35.0), (1450, 60.0)], 0),
+]
+
+
+@pytest.mark.parametrize("name,tokens,heads,in_dtype,valid,plant,knob", PLANT_CASES, ids=[c[0] for c in PLANT_CASES])
+def test_running_maximum_moves_its_reference_point_late(ctx, name, tokens, heads, in_dtype, valid, plant, knob):
+    # Keys that score 21 to 35 nats above the field sit in the first, a middle and the last key
+    # block (for the key-split shapes: in different parts), so every build of the running-maximum
+    # softmax has to move its reference point after a row's first block, rescale O and the
+    # denominator, and (where the scores arrive relative to the reference) shift the block
+    # already formed. Keys past a key limit score higher still and must stay out. Every row
+    # against the oracle on the same bf16-rounded operands; bit-identical rerun.
+    say(f"planted keys: {name}")
+    if knob == 0:
+        tail, splits = C.c_uint32(0), C.c_uint32(0)
+        hip.lib().zdraw_hip_attention_tail_plan(((tokens + 255) // 256) * heads, 256, ((valid or tokens) + 31) // 32,
+                                                C.byref(tail), C.byref(splits))
+        assert splits.value >= 3
+        per = -(-(((valid or tokens) + 31) // 32) // splits.value)  # key blocks per part
+        parts = {key // 32 // per for key, _ in plant if not valid or key < valid}
+        assert len(parts) >= 2 and max(parts) >= 2  # a later part than the first carries a planted key
+    q, k, v = _planted(tokens, heads, plant, seed=tokens + heads)
+    got = _plain_fused(ctx, q, k, v, valid=valid, in_dtype=in_dtype, knob=knob)
+    want = zo.attention_run(q, k, v, zo.Config(tokens, heads, heads, 128, False, valid))
+    mx, mean = refimpl.check_close(got, want, name)
+    say(f"  max abs {mx:.2e} mean abs {mean:.2e}")
+    # the planted keys really dominate the even rows: their output is close to the last planted V row
+    last = max((key for key, _ in plant if not valid or key < valid))
+    assert np.abs(want[0::2] - v[last][None]).max() < 0.2
+    assert np.abs(want[1::2] - v[last][None]).max() > 0.3
+    again = _plain_fused(ctx, q, k, v, valid=valid, in_dtype=in_dtype, knob=knob)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+
+
+def test_running_maximum_with_a_key_padding_mask_and_planted_keys(ctx):
+    # the boolean key mask build (block list compacted, mask words in LDS): whole blocks are
+    # dropped, planted keys sit right after a dropped stretch and inside a partly masked block
+    tokens, heads = 1024, 2
+    plant = [(10, 20.0), (330, 27.0), (700, 34.0), (200, 70.0), (650, 70.0)]
+    q, k, v = _planted(tokens, heads, plant, seed=77)
+    pad = np.zeros(tokens, np.uint8)
+    pad[128:320] = 1   # six whole blocks, key 200 among them
+    pad[640:699] = 1   # a block and most of the next, key 650 among them
+    got = _plain_fused(ctx, q, k, v, in_dtype=hip.BF16, key_pad=pad, knob=2)
+    want = zo.attention_token_list(q, k, v, zo.Config(tokens, heads, heads, 128), list(range(tokens)), key_pad=pad)
+    refimpl.check_close(got, want, "key mask with planted keys")
+    assert np.abs(want[0::2] - v[700][None]).max() < 0.2
+    again = _plain_fused(ctx, q, k, v, in_dtype=hip.BF16, key_pad=pad, knob=2)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+
+
+@pytest.mark.parametrize("k_site", [hip.K_IN_TILE_LOAD, hip.K_PREPASS])
+def test_planted_keys_through_norm_and_rope_without_a_score_bound(ctx, k_site):
+    # the fused Klein entry with norm weights far from one: the normalised scores spread over
+    # tens of nats, the caller gives no bound, and the builds that prepare K in the tile load
+    # (they subtract the reference) and in the pre-pass (scores arrive relative to it) must agree
+    # with the oracle
+    w = wl.by_name("klein_1024", seed=21, small=True)
+    rng = np.random.default_rng(3)
+    wq = (2.5 + 0.5 * rng.standard_normal(128)).astype(np.float32)
+    wk = (2.5 + 0.5 * rng.standard_normal(128)).astype(np.float32)
+    # a few keys line up with every even query of their head
+    w.k[0, 30] = w.q[0, 32] * 1.0
+    w.k[0, w.tokens - 1] = w.q[0, 34] * 1.0
+    bufs = [ctx.buffer(host.f32_to_bf16_bits(a)) for a in (w.q, w.k, w.v)]
+    o = ctx.buffer(nbytes=w.q.size * 2)
+    wb = [ctx.buffer(a) for a in (wq, wk)]
+    cos, sin = ctx.buffer(w.rope_cos), ctx.buffer(w.rope_sin)
+    ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=w.tokens, heads=w.heads, norm_q=wb[0], norm_k=wb[1],
+                    rope_cos=cos, rope_sin=sin, k_site=k_site, score_bound=0.0)
+    got = host.bf16_bits_to_f32(o.read(np.uint16, w.q.shape))[0]
+    rb = lambda a: host.bf16_bits_to_f32(host.f32_to_bf16_bits(a))
+    qn = zo.klein_apply_rope(zo.klein_rms_norm_heads(rb(w.q[0]), wq), w.rope_cos, w.rope_sin)
+    kn = zo.klein_apply_rope(zo.klein_rms_norm_heads(rb(w.k[0]), wk), w.rope_cos, w.rope_sin)
+    want = zo.attention_run(qn, kn, rb(w.v[0]), zo.Config(w.tokens, w.heads, w.heads, 128))
+    scores = np.einsum("thd,shd->hts", qn, kn) / np.sqrt(128.0)
+    assert scores.max() - np.median(scores) > 30.0  # the case is about a wide spread of scores
+    # operands rounded to bf16 after norm and rope at such score magnitudes: the probabilities are
+    # sharp, and a row's output is one V row or a close mix; the bar is the bf16 bar
+    refimpl.check_close(got, want, "klein, wide scores, no bound")
+    for b in bufs + wb + [o, cos, sin]:
+        b.release()
+
+
+def test_a_score_bound_that_is_too_small_cannot_overflow(ctx):
+    # The caller claims |q'.k'|/sqrt(128) <= 12 but the norm weights allow 11.3 * 3 * 3: the
+    # library forms the bound from the weight buffers itself and takes the running-maximum
+    # form. (With the caller's figure trusted, exp2 of the largest scores would be infinite.)
+    w = wl.by_name("klein_1024", seed=22, small=True)
+    wq = np.full(128, 3.0, np.float32)
+    wk = np.full(128, 3.0, np.float32)
+    w.k[0, 50] = w.q[0, 50]  # a key parallel to its own token's query: same rope rotation, 9 * sqrt(128) = 101 nats
+    bufs = [ctx.buffer(host.f32_to_bf16_bits(a)) for a in (w.q, w.k, w.v)]
+    wb = [ctx.buffer(a) for a in (wq, wk)]
+    cos, sin = ctx.buffer(w.rope_cos), ctx.buffer(w.rope_sin)
+    outs = []
+    for bound in (12.0, 0.0):
+        o = ctx.buffer(nbytes=w.q.size * 2)
+        ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=w.tokens, heads=w.heads, norm_q=wb[0], norm_k=wb[1],
+                        rope_cos=cos, rope_sin=sin, k_site=hip.K_PREPASS, score_bound=bound)
+        outs.append(host.bf16_bits_to_f32(o.read(np.uint16, w.q.shape))[0])
+        o.release()
+    assert np.isfinite(outs[0]).all()
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))  # the same build ran
+    # rewriting the weights through the library makes it look again
+    wb[0].write(np.full(128, 0.5, np.float32))
+    wb[1].write(np.full(128, 0.5, np.float32))
+    o = ctx.buffer(nbytes=w.q.size * 2)
+    ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=w.tokens, heads=w.heads, norm_q=wb[0], norm_k=wb[1],
+                    rope_cos=cos, rope_sin=sin, k_site=hip.K_PREPASS, score_bound=12.0)
+    small = host.bf16_bits_to_f32(o.read(np.uint16, w.q.shape))[0]
+    rb = lambda a: host.bf16_bits_to_f32(host.f32_to_bf16_bits(a))
+    half = np.full(128, 0.5, np.float32)
+    qn = zo.klein_apply_rope(zo.klein_rms_norm_heads(rb(w.q[0]), half), w.rope_cos, w.rope_sin)
+    kn = zo.klein_apply_rope(zo.klein_rms_norm_heads(rb(w.k[0]), half), w.rope_cos, w.rope_sin)
+    refimpl.check_close(small, zo.attention_run(qn, kn, rb(w.v[0]), zo.Config(w.tokens, w.heads, w.heads, 128)),
+                        "bounded after the weights were rewritten")
+    for b in bufs + wb + [o, cos, sin]:
+        b.release()
+
+
+# ------------------------------------------------------- one rope table per segment
+@pytest.mark.parametrize("k_site", [hip.K_IN_TILE_LOAD, hip.K_PREPASS])
+def test_rope_table_per_segment(ctx, k_site):
+    # klein/zflux2_resident.zig:1407-1411: the batched forward lays one rope table per image
+    # behind the other, [nb * tokens][128]; here the three tables differ (other theta, other
+    # grid split), so a segment that read a neighbour's table would be far off
+    w = wl.klein(seed=31, batch=3, heads=2, grid=(6, 7), txt_len=24, name="per-segment rope")
+    t = w.txt_len
+    tables = [zo.klein_build_rope_ref(6, 7, theta=10000.0, txt_len=t),
+              zo.klein_build_rope_ref(7, 6, theta=2000.0, txt_len=t),
+              zo.klein_build_rope_ref(3, 14, theta=500.0, txt_len=t)]
+    cos = np.concatenate([c for c, _ in tables])
+    sin = np.concatenate([s for _, s in tables])
+    assert cos.shape == (3 * w.tokens, 128)
+    rng = np.random.default_rng(4)
+    wq, wk = (1.0 + 0.2 * rng.standard_normal(128).astype(np.float32) for _ in range(2))
+    bufs = [ctx.buffer(host.f32_to_bf16_bits(a)) for a in (w.q, w.k, w.v)]
+    o = ctx.buffer(nbytes=w.q.size * 2)
+    wb = [ctx.buffer(a) for a in (wq, wk)]
+    cb, sb = ctx.buffer(cos), ctx.buffer(sin)
+    ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=w.tokens, heads=w.heads, nb=3, norm_q=wb[0], norm_k=wb[1],
+                    rope_cos=cb, rope_sin=sb, rope_per_segment=True, k_site=k_site,
+                    score_bound=host.score_bound(wq, wk))
+    got = host.bf16_bits_to_f32(o.read(np.uint16, w.q.shape))
+    cfg = zo.Config(w.tokens, w.heads, w.heads, 128)
+    wants = []
+    for b in range(3):
+        qn = zo.klein_apply_rope(zo.klein_rms_norm_heads(w.q[b], wq), *tables[b])
+        kn = zo.klein_apply_rope(zo.klein_rms_norm_heads(w.k[b], wk), *tables[b])
+        wants.append(zo.attention_run(qn, kn, w.v[b], cfg))
+        refimpl.check_close(got[b], wants[b], f"segment {b} with its own table")
+    # the tables matter: segment 1 under segment 0's table is not within the bar
+    qn = zo.klein_apply_rope(zo.klein_rms_norm_heads(w.q[1], wq), *tables[0])
+    kn = zo.klein_apply_rope(zo.klein_rms_norm_heads(w.k[1], wk), *tables[0])
+    assert np.abs(zo.attention_run(qn, kn, w.v[1], cfg) - wants[1]).max() > 5 * refimpl.MAX_ABS
+    # a table that is one row short for the last segment is refused before anything runs
+    short = ctx.buffer(cos[:-1])
+    with pytest.raises(host.InvalidShape):
+        ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=w.tokens, heads=w.heads, nb=3, norm_q=wb[0],
+                        norm_k=wb[1], rope_cos=short, rope_sin=sb, rope_per_segment=True, k_site=k_site)
+    for b in bufs + wb + [o, cb, sb, short]:
+        b.release()
+
+
+# ------------------------------- standalone QK-norm + rope: Klein in place, reference form
+def _qk_pipeline(ctx):
+    err = C.create_string_buffer(128)
+    pipe = hip.lib().zdraw_hip_compile(ctx.device, b"// shader text is not read", b"qk_norm_rope", err, 128)
+    assert pipe, err.value
+    return pipe
+
+
+def test_klein_krms_rope_in_place_matches_oracle(ctx):
+    # klein/zflux2_resident.zig:1573-1579 (rmsRope): krms_rope in place on f32 token-major rows,
+    # text rows under the added-stream weights; q and k have different head counts here
+    L = hip.lib()
+    rng = np.random.default_rng(12)
+    tokens, heads, kv_heads, t = 75, 5, 3, 20
+    q = rng.standard_normal((tokens, heads, 128), dtype=np.float32)
+    k = rng.standard_normal((tokens, kv_heads, 128), dtype=np.float32)
+    wq, wk, wqt, wkt = (1.0 + 0.3 * rng.standard_normal(128).astype(np.float32) for _ in range(4))
+    cos, sin = zo.klein_build_rope_ref(5, 11, theta=2000.0, txt_len=t)
+    assert cos.shape[0] == tokens
+    qb, kb = ctx.buffer(q), ctx.buffer(k)
+    wb = [ctx.buffer(a) for a in (wq, wk, wqt, wkt)]
+    cb, sb = ctx.buffer(cos), ctx.buffer(sin)
+    pipe = _qk_pipeline(ctx)
+    p = hip.AttnParams(tokens, heads, kv_heads, 128, 0, 0)
+    x = hip.AttnExt()
+    x.qk_mode, x.eps, x.txt_rows = hip.QK_KLEIN, wl.KLEIN_EPS, t
+    ops = hip.QkOperands()
+    ops.q_weight, ops.k_weight, ops.q_weight_txt, ops.k_weight_txt = (b.handle for b in wb)
+    ops.rope_cos, ops.rope_sin = cb.handle, sb.handle
+    d0 = L.zdraw_hip_dispatch_count()
+    rc = L.zdraw_hip_run_qk_norm_rope_ext(ctx.queue, pipe, qb.handle, kb.handle, C.byref(p), C.byref(x), C.byref(ops))
+    assert rc == 0, hip.last_error()
+    assert L.zdraw_hip_dispatch_count() - d0 == 2
+    gq, gk = qb.read(np.float32, q.shape), kb.read(np.float32, k.shape)
+    for got, x0, w_img, w_txt in ((gq, q, wq, wqt), (gk, k, wk, wkt)):
+        n = np.concatenate([zo.klein_rms_norm_heads(x0[:t], w_txt), zo.klein_rms_norm_heads(x0[t:], w_img)])
+        want = zo.klein_apply_rope(n, cos, sin)
+        # fp32 on both sides; the oracle sums the squares in f64 and divides, the kernel in f32 with rsqrt
+        assert np.abs(got - want).max() < 5e-6 * np.abs(want).max() + 2e-6
+    # a wrong pipeline kind is a handle error, nothing runs
+    assert L.zdraw_hip_run_qk_norm_rope_ext(ctx.queue, ctx.block_pipeline, qb.handle, kb.handle, C.byref(p), C.byref(x),
+                                            C.byref(ops)) == hip.ERR_HANDLE
+    L.zdraw_hip_release_pipeline(pipe)
+    for b in [qb, kb, cb, sb] + wb:
+        b.release()
+
+
+@pytest.mark.parametrize("wname", ["f32", "bf16", "f16"])
+def test_qk_norm_rope_in_the_reference_argument_form(ctx, wname):
+    # metal_c.zig:148-159 as mqk.run issues it (metal/mqk.zig:37-57): buffers for q, k, both
+    # weights, positions and the pair table, QkNormParams with the weights' type and byte
+    # offsets, a thread count. Against the oracle; then positions outside the table.
+    L = hip.lib()
+    rng = np.random.default_rng(13)
+    tokens, heads, kv_heads = 70, 4, 2
+    cfg = zo.RopeConfig(wl.ZIMAGE_DIMS, wl.ZIMAGE_LENS, wl.ZIMAGE_THETA)
+    vals = zo.zrope_fill(cfg)
+    bases = zo.zrope_axis_bases(cfg)
+    pos = np.stack([rng.integers(0, 1536, tokens), rng.integers(0, 512, tokens), rng.integers(0, 512, tokens)], 1).astype(np.uint64)
+    pos[0] = (1535, 511, 511)  # the last entry of every axis
+    q = rng.standard_normal((tokens, heads, 128), dtype=np.float32)
+    k = rng.standard_normal((tokens, kv_heads, 128), dtype=np.float32)
+    wq = (1.0 + 0.2 * rng.standard_normal(128)).astype(np.float32)
+    wk = (1.0 + 0.2 * rng.standard_normal(128)).astype(np.float32)
+    if wname == "f32":
+        code, enc, dec = hip.W_F32, (lambda a: a.astype(np.float32)), (lambda a: a)
+    elif wname == "bf16":
+        code, enc, dec = hip.W_BF16, host.f32_to_bf16_bits, host.bf16_bits_to_f32
+    else:
+        code, enc, dec = hip.W_F16, (lambda a: a.astype(np.float16)), (lambda a: a.astype(np.float32))
+    # both weights in one buffer at byte offsets, as a view into a checkpoint would be
+    q_off, k_off = 64, 64 + 512
+    blob = np.zeros(2048, np.uint8)
+    eq, ek = enc(wq), enc(wk)
+    blob[q_off:q_off + eq.nbytes] = eq.view(np.uint8)
+    blob[k_off:k_off + ek.nbytes] = ek.view(np.uint8)
+    wq_used, wk_used = dec(eq), dec(ek)
+    weights = ctx.buffer(blob)
+    posb, ropeb = ctx.buffer(pos), ctx.buffer(vals)
+    pipe = _qk_pipeline(ctx)
+    qp = hip.QkNormParams(tokens, heads, kv_heads, 128, code, code, *wl.ZIMAGE_DIMS, wl.ZIMAGE_EPS, q_off, k_off, *bases)
+
+    def run(positions):
+        posb.write(np.ascontiguousarray(positions, np.uint64))
+        qb, kb = ctx.buffer(q), ctx.buffer(k)
+        rc = L.zdraw_hip_run_qk_norm_rope(ctx.queue, pipe, qb.handle, kb.handle, weights.handle, weights.handle,
+                                          posb.handle, ropeb.handle, C.byref(qp), 256)
+        assert rc == 0, hip.last_error()
+        out = qb.read(np.float32, q.shape), kb.read(np.float32, k.shape)
+        qb.release()
+        kb.release()
+        return out
+
+    gq, gk = run(pos)
+    want_q = zo.zimage_rotate(zo.zimage_norm_heads(q, wq_used, wl.ZIMAGE_EPS), vals, cfg, pos.astype(np.uintp))
+    want_k = zo.zimage_rotate(zo.zimage_norm_heads(k, wk_used, wl.ZIMAGE_EPS), vals, cfg, pos.astype(np.uintp))
+    assert np.abs(gq - want_q).max() < 5e-6 * np.abs(want_q).max() + 2e-6
+    assert np.abs(gk - want_k).max() < 5e-6 * np.abs(want_k).max() + 2e-6
+    # positions at or past an axis's length (zimage/zrope.zig:48 refuses them where the host sees
+    # them): the call completes, such a token is rotated by its axis's last table entry, every
+    # other token keeps its bits
+    bad = pos.copy()
+    bad[5] = (1536, 3, 4)
+    bad[6] = (7, 2 ** 40, 9)
+    bad[7] = (1, 2, 2 ** 63)
+    held = pos.copy()
+    held[5] = (1535, 3, 4)
+    held[6] = (7, 511, 9)
+    held[7] = (1, 2, 511)
+    bq, bk = run(bad)
+    hq, hk = run(held)
+    assert np.array_equal(bq.view(np.uint32), hq.view(np.uint32)) and np.array_equal(bk.view(np.uint32), hk.view(np.uint32))
+    keep = np.ones(tokens, bool)
+    keep[5:8] = False
+    assert np.array_equal(bq[keep].view(np.uint32), gq[keep].view(np.uint32))
+    # malformed calls are refused before anything runs
+    d0 = L.zdraw_hip_dispatch_count()
+    bad_qp = hip.QkNormParams(tokens, heads, kv_heads, 128, code, code, 32, 48, 40, wl.ZIMAGE_EPS, q_off, k_off, *bases)
+    qb = ctx.buffer(q)
+    assert L.zdraw_hip_run_qk_norm_rope(ctx.queue, pipe, qb.handle, qb.handle, weights.handle, weights.handle,
+                                        posb.handle, ropeb.handle, C.byref(bad_qp), 256) == hip.INVALID
+    far = hip.QkNormParams(tokens, heads, kv_heads, 128, code, code, *wl.ZIMAGE_DIMS, wl.ZIMAGE_EPS, 4096, k_off, *bases)
+    assert L.zdraw_hip_run_qk_norm_rope(ctx.queue, pipe, qb.handle, qb.handle, weights.handle, weights.handle,
+                                        posb.handle, ropeb.handle, C.byref(far), 256) == hip.INVALID
+    assert L.zdraw_hip_dispatch_count() == d0
+    qb.release()
+    L.zdraw_hip_release_pipeline(pipe)
+    for b in (weights, posb, ropeb):
+        b.release()
+
+
+def test_fused_zimage_entry_holds_device_positions_to_the_table(ctx):
+    # the fused entry carries no axis lengths: it derives them from the pair table's size, and a
+    # position past an axis reads the axis's last entry instead of memory outside the table
+    w = wl.by_name("zimage_1024", seed=9, small=True)
+    outs = []
+    for variant in ("bad", "held"):
+        pos = np.ascontiguousarray(w.pos, np.uint64).copy()
+        pos[3] = (2 ** 33, 1, 2) if variant == "bad" else (1535, 1, 2)
+        pos[40] = (3, 512, 700) if variant == "bad" else (3, 511, 511)
+        for k_site in (hip.K_PREPASS, hip.K_IN_TILE_LOAD):
+            res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=k_site)
+            res.pos.write(pos)
+            outs.append(res.run())
+            res.release()
+    assert np.isfinite(outs[0]).all()
+    assert np.array_equal(outs[0].view(np.uint32), outs[2].view(np.uint32))
+    assert np.array_equal(outs[1].view(np.uint32), outs[3].view(np.uint32))

@@ -30,7 +30,7 @@ def ctx():
 def pipe(ctx):
     L = hip.lib()
     err = C.create_string_buffer(128)
-    p = L.zdraw_hip_compile(ctx.device, b"gemm_half", err, 128)
+    p = L.zdraw_hip_compile(ctx.device, None, b"gemm_half", err, 128)
     assert p, err.value
     yield p
     L.zdraw_hip_release_pipeline(p)

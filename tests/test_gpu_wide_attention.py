@@ -100,7 +100,7 @@ def test_wide_head_refusals_leave_nothing_enqueued(ctx):
     assert L.zdraw_hip_dispatch_count() == d0
     # C ABI: the wide pipeline runs kernel = wide only, and the block pipeline refuses width 512
     err = C.create_string_buffer(128)
-    wide = L.zdraw_hip_compile(ctx.device, b"attention_wide_mfma", err, 128)
+    wide = L.zdraw_hip_compile(ctx.device, None, b"attention_wide_mfma", err, 128)
     assert wide, err.value
     assert L.zdraw_hip_pipeline_threads(wide) == 512
     b = ctx.buffer(z4)
@@ -129,7 +129,7 @@ def test_wide_head_batch_offsets(ctx):
     qb, kb, vb = ctx.buffer(q), ctx.buffer(k), ctx.buffer(v)
     ob = ctx.buffer(nbytes=q.nbytes)
     err = C.create_string_buffer(128)
-    wide = L.zdraw_hip_compile(ctx.device, b"attention_wide_mfma", err, 128)
+    wide = L.zdraw_hip_compile(ctx.device, None, b"attention_wide_mfma", err, 128)
     p = hip.AttnParams(tokens, 1, 1, 512, 0, 0)
     seg = tokens * 512 * 4
     batch = L.zdraw_hip_batch_begin(ctx.queue)

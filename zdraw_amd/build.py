@@ -43,7 +43,7 @@ def build_hip(verbose: bool = False, out: str | None = None, extra_flags=()) -> 
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     target = out or HIP_LIB
     tag = "" if out is None else "." + os.path.basename(out)
-    srcs = [os.path.join(CSRC, f) for f in ("attn_fwd.hip", "attn_wide.hip", "qk_prepass.hip", "gemm_half.hip", "mfma_probe.hip", "bridge.hip")]
+    srcs = [os.path.join(CSRC, f) for f in ("attn_fwd.hip", "attn_wide.hip", "qk_prepass.hip", "gemm_half.hip", "bridge.hip")]
     objs = []
     for src in srcs:
         obj = os.path.join(LIBDIR, os.path.basename(src) + tag + ".o")

@@ -187,13 +187,18 @@ __device__ __forceinline__ Rope8 ld_rope8(const QkOps& a, int mode, const QkRow&
         // launch arguments and parks the positions in scratch.
         const int dim0 = a.dim0, dim1 = a.dim1, dim2 = a.dim2;
         const unsigned base0 = a.base0, base1 = a.base1, base2 = a.base2;
+        const unsigned len0 = a.len0, len1 = a.len1, len2 = a.len2;
         const unsigned long long q0 = r.p0, q1 = r.p1, q2 = r.p2;
         const int d01 = dim0 + dim1;
         const int axis = d0 < dim0 ? 0 : (d0 < d01 ? 1 : 2);
         const int axis_off = axis == 0 ? 0 : (axis == 1 ? dim0 : d01);
         const unsigned axis_pairs = (unsigned)(axis == 0 ? dim0 : (axis == 1 ? dim1 : dim2)) >> 1;
         const unsigned base = axis == 0 ? base0 : (axis == 1 ? base1 : base2);
-        const unsigned long long p = axis == 0 ? q0 : (axis == 1 ? q1 : q2);
+        const unsigned long long p_raw = axis == 0 ? q0 : (axis == 1 ? q1 : q2);
+        // zimage/zrope.zig:48 refuses pos >= len on the host; a device-resident position is
+        // held to the table instead (the axis's last entry)
+        const unsigned last = (axis == 0 ? len0 : (axis == 1 ? len1 : len2)) - 1u;
+        const unsigned long long p = p_raw < (unsigned long long)last ? p_raw : (unsigned long long)last;
         const unsigned long long idx = base + p * axis_pairs + (unsigned)((d0 - axis_off) >> 1);
         const float* src = a.pairs + idx * 2;
         t.a = *reinterpret_cast<const f32x4*>(src);      // (c0,s0,c1,s1)

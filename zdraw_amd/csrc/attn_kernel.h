@@ -29,6 +29,9 @@ struct QkOps {
     int64_t rope_bs;    // table / position rows between segments (0 = shared)
     uint32_t base0, base1, base2; // Z-Image axis bases in pairs
     int32_t dim0, dim1, dim2;     // Z-Image axis widths
+    // Z-Image: positions the pair table holds per axis (>= 1); a position at or past its
+    // axis's count reads the axis's last entry, so no position can index outside the table
+    uint32_t len0, len1, len2;
     int32_t txt_rows;   // tokens < txt_rows use the *_txt weights when given
     float eps;
 };

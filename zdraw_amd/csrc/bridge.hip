@@ -8,6 +8,7 @@
 // before a kernel is launched, because a kernel that reads out of bounds can
 // take the whole device down.
 #include "../../include/zdraw_hip.h"
+#include "../../include/zdraw_hip_measure.h"
 #include "attn_kernel.h"
 #include "gemm_kernel.h"
 
@@ -166,6 +167,20 @@ bool need(const void* handle, size_t bytes) {
     return b && b->ptr && b->len >= bytes && ((uintptr_t)b->ptr % 16) == 0;
 }
 
+// Where a call's scratch comes from: the library's grow-only slots (zdraw_hip_attn_scratch),
+// or a caller-supplied span handed out piece by piece in 256-byte steps (the entry that
+// allocates nothing), or nowhere (a plan that is only validated).
+struct ScratchSource {
+    Device* dev;
+    bool dry;
+    char* span = nullptr; // bump allocation over [span, span + cap)
+    size_t cap = 0, used = 0;
+    bool over = false;    // the span was too small for what the call needs
+    ScratchSource(Device* d, bool dry_run = false) : dev(d), dry(dry_run) {}
+    ScratchSource(Device* d, void* base, size_t bytes) : dev(d), dry(false), span(static_cast<char*>(base)), cap(bytes) {}
+    void* get(int slot, size_t bytes);
+};
+
 constexpr uint32_t kRoundPlainTokens = 1024; // plain f32 attention from this length on rounds its operands once, ahead of the kernel
 
 struct FusedPlan {
@@ -192,11 +207,97 @@ int norm_weight_dtype(uint32_t coded) {
     return coded == ZDRAW_HIP_W_F32 ? (int)kF32 : coded == ZDRAW_HIP_W_F16 ? (int)kF16 : coded == ZDRAW_HIP_W_BF16 ? (int)kBF16 : -1;
 }
 
+// max |w| over the 128 norm weights at `off` in `b`, element type `dtype` (kF32, kF16, kBF16).
+// The weights live on the device: they are read back once per (address, type) and the figure is
+// kept until the buffer is written through this library or released. +inf if they cannot be
+// read or hold a NaN (the caller then gets the running-maximum softmax).
+struct WeightMax {
+    const void* ptr;
+    int dtype;
+    float amax;
+};
+std::vector<WeightMax> g_weight_max;
+
+void forget_weight_max(const Buffer* b) {
+    const char* lo = static_cast<const char*>(b->ptr);
+    const char* hi = lo + b->len;
+    for (size_t i = 0; i < g_weight_max.size();) {
+        const char* p = static_cast<const char*>(g_weight_max[i].ptr);
+        if (p >= lo && p < hi) {
+            g_weight_max[i] = g_weight_max.back();
+            g_weight_max.pop_back();
+        } else {
+            i++;
+        }
+    }
+}
+
+float weight_abs_max(const Buffer* b, uint64_t off, int dtype) {
+    const void* src = static_cast<const char*>(b->ptr) + off;
+    for (const WeightMax& w : g_weight_max)
+        if (w.ptr == src && w.dtype == dtype) return w.amax;
+    unsigned char raw[kHeadDim * 4];
+    const size_t bytes = (size_t)kHeadDim * (dtype == kF32 ? 4 : 2);
+    if (hipMemcpy(raw, src, bytes, hipMemcpyDeviceToHost) != hipSuccess) return INFINITY;
+    float m = 0.f;
+    for (int i = 0; i < kHeadDim; i++) {
+        float v;
+        if (dtype == kF32) {
+            memcpy(&v, raw + 4 * i, 4);
+        } else {
+            uint16_t h;
+            memcpy(&h, raw + 2 * i, 2);
+            if (dtype == kBF16) {
+                const uint32_t u = (uint32_t)h << 16;
+                memcpy(&v, &u, 4);
+            } else {
+                v = (float)__builtin_bit_cast(_Float16, h);
+            }
+        }
+        v = fabsf(v);
+        if (!(v <= m)) m = v; // a NaN sticks
+    }
+    if (!(m >= 0.0f)) m = INFINITY;
+    if (g_weight_max.size() >= 256) g_weight_max.clear();
+    g_weight_max.push_back(WeightMax{src, dtype, m});
+    return m;
+}
+
+// How many positions of each Z-Image rope axis lie inside a (cos,sin) pair table of
+// `table_bytes` bytes: axis i holds dims[i] / 2 pairs per position from pair base[i] up to the
+// next axis base above it (or the end of the table). The layout of zrope.Cache
+// (zimage/zrope.zig:29-42, 118-140) gives back its `lens`. False when an axis has no whole
+// position inside the table.
+bool zimage_axis_lens(uint64_t table_bytes, const uint64_t base[3], const uint32_t dims[3], uint32_t lens[3]) {
+    const uint64_t total = table_bytes / 8; // pairs
+    for (int i = 0; i < 3; i++) {
+        const uint64_t per = dims[i] / 2;
+        if (per == 0 || base[i] >= total) return false;
+        uint64_t end = total;
+        for (int j = 0; j < 3; j++)
+            if (base[j] > base[i] && base[j] < end) end = base[j];
+        const uint64_t n = (end - base[i]) / per;
+        if (n == 0) return false;
+        lens[i] = n > 0xffffffffull ? 0xffffffffu : (uint32_t)n;
+    }
+    return true;
+}
+
 // Shared validation + argument assembly. Returns 0 or an ABI return code.
 // nw == nullptr: norm weights are f32[128] at offset 0.
+int scratch_failed(const ScratchSource* src) {
+    if (src->over) {
+        g_fallback++;
+        set_err("unavailable: the call needs more than the %zu bytes of scratch this entry holds", src->cap);
+        return ZDRAW_HIP_UNAVAILABLE;
+    }
+    set_err("scratch allocation failed");
+    return ZDRAW_HIP_ERR_HANDLE;
+}
+
 int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const ZdrawAttnParams* p,
                    const ZdrawHipAttnExt* x, const ZdrawHipQkOperands* ops, FusedPlan* plan,
-                   const NormWeights* nw = nullptr) {
+                   ScratchSource* src, const NormWeights* nw = nullptr) {
     if (!p || !x) {
         set_err("null params");
         return ZDRAW_HIP_ERR_HANDLE;
@@ -245,10 +346,8 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     a.q_mode = (int32_t)x->qk_mode;
     a.out_dtype = (int32_t)x->out_dtype;
     a.scale_log2 = 1.4426950408889634f / sqrtf((float)kHeadDim);
-    // exp2 of a scaled score must stay far from the fp32 exponent limits: 2^64 times
-    // tokens (<= 2^15) times |v| still fits, 2^-64 does not underflow
     if (!(x->score_bound >= 0.0f)) return invalid("score_bound");
-    a.bounded = (x->score_bound > 0.0f && x->score_bound * 1.4426950408889634f <= 64.0f) ? 1 : 0;
+    float bound = x->score_bound; // raised below to what the norm weights themselves allow
     if ((int64_t)a.nqb * a.heads * a.batch > 0x7fffffffLL) return unavailable("grid too large");
 
     const uint64_t rows_needed = (uint64_t)(x->batch - 1) * x->rope_batch_rows + p->tokens;
@@ -284,6 +383,19 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         a.qk.txt_rows = (int32_t)x->txt_rows;
         a.qk.eps = x->eps;
         a.qk.rope_bs = (int64_t)x->rope_batch_rows;
+        if (bound > 0.0f) {
+            // The caller asks for the form without a running maximum. Whether the scores allow it
+            // is a function of the norm weights alone (rows normalised to sqrt(128) max|w|, a rope
+            // that rotates): the library forms that bound itself, so a caller's figure that is too
+            // small cannot make the exponentials overflow.
+            float mq = weight_abs_max(static_cast<Buffer*>(ops->q_weight), qwo, qwd);
+            float mk = weight_abs_max(static_cast<Buffer*>(ops->k_weight), kwo, kwd);
+            if (ops->q_weight_txt) mq = fmaxf(mq, weight_abs_max(static_cast<Buffer*>(ops->q_weight_txt), 0, kF32));
+            if (ops->k_weight_txt) mk = fmaxf(mk, weight_abs_max(static_cast<Buffer*>(ops->k_weight_txt), 0, kF32));
+            const float own = sqrtf((float)kHeadDim) * mq * mk * 1.02f; // 2 % for the roundings of norm and operands
+            bound = (own >= bound) ? own : bound;                       // a NaN or infinite weight: no bound
+            if (!(own >= 0.0f)) bound = INFINITY;
+        }
         if (x->qk_mode == ZDRAW_HIP_QK_KLEIN) {
             const size_t bytes = (size_t)rows_needed * kHeadDim * 4;
             if (!need(ops->rope_cos, bytes) || !need(ops->rope_sin, bytes))
@@ -300,10 +412,11 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
                     return unavailable("zimage axis bases must be even and fit 32 bits");
             if (!need(ops->pos, (size_t)rows_needed * 24)) return invalid("positions too small for [rows][3] u64");
             if (!need(ops->rope_pairs, 16)) return invalid("rope pair table missing");
-            // every axis must have at least one position's worth of pairs inside the table
+            // positions per axis that lie inside the table: the kernels hold every position to them
             const Buffer* pt = static_cast<Buffer*>(ops->rope_pairs);
-            for (int i = 0; i < 3; i++)
-                if ((x->zimage_base[i] + d[i] / 2) * 8 > pt->len) return invalid("rope pair table smaller than an axis base");
+            uint32_t lens[3];
+            if (!zimage_axis_lens(pt->len, x->zimage_base, d, lens)) return invalid("rope pair table smaller than an axis base");
+            a.qk.len0 = lens[0]; a.qk.len1 = lens[1]; a.qk.len2 = lens[2];
             a.qk.pos = static_cast<const unsigned long long*>(static_cast<Buffer*>(ops->pos)->ptr);
             a.qk.pairs = static_cast<const float*>(pt->ptr);
             a.qk.dim0 = (int32_t)d[0]; a.qk.dim1 = (int32_t)d[1]; a.qk.dim2 = (int32_t)d[2];
@@ -312,6 +425,9 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
             a.qk.base2 = (uint32_t)x->zimage_base[2];
         }
     }
+    // exp2 of a scaled score must stay far from the fp32 exponent limits: 2^64 times
+    // tokens (<= 2^15) times |v| still fits, 2^-64 does not underflow
+    a.bounded = (bound > 0.0f && bound * 1.4426950408889634f <= 64.0f) ? 1 : 0;
     if (ops && ops->key_pad) {
         const Buffer* m = static_cast<Buffer*>(ops->key_pad);
         const uint64_t mbytes = (uint64_t)(x->batch - 1) * x->mask_batch_bytes + p->tokens;
@@ -327,16 +443,13 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         attention_tail_plan((int64_t)a.nqb * a.heads * a.batch, dev->cus, (a.key_limit + attention_key_block() - 1) / attention_key_block(),
                             &tail, &splits);
         if (splits > 1) {
-            Buffer* po = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 3, attention_part_o_bytes(tail, splits, g_variant & 1)));
-            Buffer* pm = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 4, attention_part_ml_bytes(tail, splits, g_variant & 1)));
-            if (!po || !pm) {
-                set_err("scratch allocation failed");
-                return ZDRAW_HIP_ERR_HANDLE;
-            }
+            void* po = src->get(3, attention_part_o_bytes(tail, splits, g_variant & 1));
+            void* pm = src->get(4, attention_part_ml_bytes(tail, splits, g_variant & 1));
+            if (!po || !pm) return scratch_failed(src);
             a.splits = splits;
             a.tile_base = tail; // launch_attention reads the tail size here
-            a.part_o = static_cast<float*>(po->ptr);
-            a.part_ml = static_cast<float*>(pm->ptr);
+            a.part_o = static_cast<float*>(po);
+            a.part_ml = static_cast<float*>(pm);
         }
     }
     plan->args = a;
@@ -357,12 +470,9 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         const uint32_t prep_out = to_bf16 ? (uint32_t)ZDRAW_HIP_BF16 : x->in_dtype;
         const size_t es = elem_size(prep_out);
         const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * es;
-        Buffer* sq = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 0, bytes));
-        Buffer* sk = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 1, bytes));
-        if (!sq || !sk) {
-            set_err("scratch allocation failed");
-            return ZDRAW_HIP_ERR_HANDLE;
-        }
+        void* sq = src->get(0, bytes);
+        void* sk = src->get(1, bytes);
+        if (!sq || !sk) return scratch_failed(src);
         PrepArgs pr;
         memset(&pr, 0, sizeof(pr));
         pr.y_bs = (int64_t)p->heads * p->tokens * kHeadDim;
@@ -375,13 +485,13 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         pr.w_dtype = plan->w_dtype;
         PrepArgs pq = pr;
         pr.x = a.k;
-        pr.y = sk->ptr;
+        pr.y = sk;
         pr.x_bs = a.k_bs; pr.x_ts = a.k_ts; pr.x_hs = a.k_hs;
         pr.w = a.k_w;
         pr.w_txt = a.k_w_txt;
         pr.scale = 1.0f;
         pq.x = a.q;
-        pq.y = sq->ptr;
+        pq.y = sq;
         pq.x_bs = a.q_bs; pq.x_ts = a.q_ts; pq.x_hs = a.q_hs;
         pq.w = a.q_w;
         pq.w_txt = a.q_w_txt;
@@ -390,29 +500,26 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         plan->prep_q = pq;
         plan->prepass = true;
         plan->k_mode = kQkNone;
-        plan->args.k = sk->ptr;
+        plan->args.k = sk;
         plan->args.k_bs = pr.y_bs; plan->args.k_ts = pr.y_ts; plan->args.k_hs = pr.y_hs;
-        plan->args.q = sq->ptr;
+        plan->args.q = sq;
         plan->args.q_bs = pr.y_bs; plan->args.q_ts = pr.y_ts; plan->args.q_hs = pr.y_hs;
         plan->args.q_mode = kQkNone;
         plan->args.scale_log2 = 1.0f;
         plan->prep_in_dtype = (int)x->in_dtype;
         if (to_bf16) {
-            Buffer* sv = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, 2, bytes));
-            if (!sv) {
-                set_err("scratch allocation failed");
-                return ZDRAW_HIP_ERR_HANDLE;
-            }
+            void* sv = src->get(2, bytes);
+            if (!sv) return scratch_failed(src);
             PrepArgs pv = pr;
             pv.mode = kQkNone;
             pv.x = a.v;
-            pv.y = sv->ptr;
+            pv.y = sv;
             pv.x_bs = a.v_bs; pv.x_ts = a.v_ts; pv.x_hs = a.v_hs;
             pv.w = pv.w_txt = nullptr;
             pv.scale = 1.0f;
             plan->prep_v = pv;
             plan->round_v = true;
-            plan->args.v = sv->ptr;
+            plan->args.v = sv;
             plan->args.v_bs = pr.y_bs; plan->args.v_ts = pr.y_ts; plan->args.v_hs = pr.y_hs;
             plan->in_dtype = kBF16;
         }
@@ -423,13 +530,10 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         // slots 0-2 by one launch, and the kernel is the direct-to-LDS build, as for prepared
         // operands. Short sequences stay on the build that rounds in its tile load.
         const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * 2;
-        Buffer* sc[3];
+        void* sc[3];
         for (int i = 0; i < 3; i++) {
-            sc[i] = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, i, bytes));
-            if (!sc[i]) {
-                set_err("scratch allocation failed");
-                return ZDRAW_HIP_ERR_HANDLE;
-            }
+            sc[i] = src->get(i, bytes);
+            if (!sc[i]) return scratch_failed(src);
         }
         PrepArgs pr;
         memset(&pr, 0, sizeof(pr));
@@ -441,9 +545,9 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         pr.out_dtype = kBF16;
         pr.scale = 1.0f;
         PrepArgs pq = pr, pk = pr, pv = pr;
-        pq.x = a.q; pq.y = sc[0]->ptr; pq.x_bs = a.q_bs; pq.x_ts = a.q_ts; pq.x_hs = a.q_hs; pq.scale = a.scale_log2;
-        pk.x = a.k; pk.y = sc[1]->ptr; pk.x_bs = a.k_bs; pk.x_ts = a.k_ts; pk.x_hs = a.k_hs;
-        pv.x = a.v; pv.y = sc[2]->ptr; pv.x_bs = a.v_bs; pv.x_ts = a.v_ts; pv.x_hs = a.v_hs;
+        pq.x = a.q; pq.y = sc[0]; pq.x_bs = a.q_bs; pq.x_ts = a.q_ts; pq.x_hs = a.q_hs; pq.scale = a.scale_log2;
+        pk.x = a.k; pk.y = sc[1]; pk.x_bs = a.k_bs; pk.x_ts = a.k_ts; pk.x_hs = a.k_hs;
+        pv.x = a.v; pv.y = sc[2]; pv.x_bs = a.v_bs; pv.x_ts = a.v_ts; pv.x_hs = a.v_hs;
         plan->prep_q = pq;
         plan->prep = pk;
         plan->prep_v = pv;
@@ -451,9 +555,9 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         plan->prepass = true;
         plan->prep_in_dtype = kF32;
         plan->in_dtype = kBF16;
-        plan->args.q = sc[0]->ptr;
-        plan->args.k = sc[1]->ptr;
-        plan->args.v = sc[2]->ptr;
+        plan->args.q = sc[0];
+        plan->args.k = sc[1];
+        plan->args.v = sc[2];
         plan->args.q_bs = plan->args.k_bs = plan->args.v_bs = pr.y_bs;
         plan->args.q_ts = plan->args.k_ts = plan->args.v_ts = pr.y_ts;
         plan->args.q_hs = plan->args.k_hs = plan->args.v_hs = pr.y_hs;
@@ -625,6 +729,21 @@ int finish_blocking(Queue* qu, hipEvent_t start, hipEvent_t stop) {
 }
 
 Buffer* g_scratch[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+
+void* ScratchSource::get(int slot, size_t bytes) {
+    if (dry) return reinterpret_cast<void*>(uintptr_t{256}); // never dereferenced: the plan is not launched
+    if (span) {
+        const size_t at = (used + 255) & ~size_t{255};
+        if (bytes > cap || at > cap - bytes) {
+            over = true;
+            return nullptr;
+        }
+        used = at + bytes;
+        return span + at;
+    }
+    Buffer* b = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, slot, bytes));
+    return b ? b->ptr : nullptr;
+}
 
 bool scratch_poisoned(int slot) {
     // ZDRAW_SCRATCH_POISON: "1" every slot, "attn" the group, "attn:2" one slot
@@ -843,6 +962,7 @@ void zdraw_hip_read_buffer(void* buffer, uint8_t* dst, size_t size) {
 void zdraw_hip_write_buffer(void* buffer, const uint8_t* src, size_t size) {
     Buffer* b = static_cast<Buffer*>(buffer);
     if (!b || !src || size > b->len) return;
+    forget_weight_max(b);
     (void)hipMemcpy(b->ptr, src, size, hipMemcpyHostToDevice);
 }
 
@@ -859,12 +979,14 @@ void* zdraw_hip_buffer_device_ptr(void* buffer) {
 void zdraw_hip_release_buffer(void* buffer) {
     Buffer* b = static_cast<Buffer*>(buffer);
     if (!b) return;
+    if (b->ptr) forget_weight_max(b);
     if (b->owned && b->ptr) (void)hipFree(b->ptr);
     delete b;
 }
 
 // ---------------------------------------------------------------- pipelines
-void* zdraw_hip_compile(void* device, const char* entry, char* error_buf, size_t error_len) {
+void* zdraw_hip_compile(void* device, const char* source, const char* entry, char* error_buf, size_t error_len) {
+    (void)source; // the kernels were compiled ahead of time; the reference's call sites pass their shader text here
     if (error_buf && error_len) error_buf[0] = '\0';
     if (!device || !entry) return nullptr;
     if (strcmp(entry, "attention_block_mfma") == 0) return new Pipeline{0};
@@ -900,7 +1022,8 @@ int zdraw_hip_run_attention(void* queue, void* pipeline, void* q, void* k, void*
     FusedPlan plan;
     if (!wide) {
         standalone_ext(params, 0, 0, &x);
-        rc = plan_attention(qu->dev, q, k, v, output, params, &x, nullptr, &plan);
+        ScratchSource slots(qu->dev);
+        rc = plan_attention(qu->dev, q, k, v, output, params, &x, nullptr, &plan, &slots);
         if (rc != ZDRAW_HIP_OK) return rc;
     }
     hipEvent_t start, stop;
@@ -941,7 +1064,8 @@ int zdraw_hip_run_attention_enc_off(void* batch, void* pipeline, void* q, void* 
     ZdrawHipAttnExt x;
     standalone_ext(params, in_off, out_off, &x);
     FusedPlan plan;
-    rc = plan_attention(b->queue->dev, q, k, v, o, params, &x, nullptr, &plan);
+    ScratchSource slots(b->queue->dev);
+    rc = plan_attention(b->queue->dev, q, k, v, o, params, &x, nullptr, &plan, &slots);
     if (rc != ZDRAW_HIP_OK) return rc;
     return enqueue(plan, b->queue->stream);
 }
@@ -970,7 +1094,8 @@ int zdraw_hip_run_attention_fused_enc(void* batch, void* q, void* k, void* v, vo
         return ZDRAW_HIP_ERR_HANDLE;
     }
     FusedPlan plan;
-    int rc = plan_attention(b->queue->dev, q, k, v, out, params, ext, ops, &plan);
+    ScratchSource slots(b->queue->dev);
+    int rc = plan_attention(b->queue->dev, q, k, v, out, params, ext, ops, &plan, &slots);
     if (rc != ZDRAW_HIP_OK) return rc;
     return enqueue(plan, b->queue->stream);
 }
@@ -988,9 +1113,11 @@ int zdraw_hip_run_attention_fused(void* queue, void* q, void* k, void* v, void* 
     return rc != ZDRAW_HIP_OK ? rc : rc2;
 }
 
-int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
-                               const ZdrawAttnParams* p, const ZdrawHipAttnExt* x,
-                               const ZdrawHipQkOperands* ops) {
+namespace {
+// In-place norm + rope of q (then k) on f32 token-major rows: one pre-pass launch each.
+// nw == nullptr: norm weights are f32[128] at offset 0.
+int run_qk_norm_rope_impl(void* queue, void* pipeline, void* q, void* k, const ZdrawAttnParams* p,
+                          const ZdrawHipAttnExt* x, const ZdrawHipQkOperands* ops, const NormWeights* nw) {
     Queue* qu = static_cast<Queue*>(queue);
     if (!qu || !p || !x || !ops) {
         set_err("null argument");
@@ -1004,15 +1131,18 @@ int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
     if (x->qk_mode != ZDRAW_HIP_QK_KLEIN && x->qk_mode != ZDRAW_HIP_QK_ZIMAGE) return invalid("qk_mode");
     // Reuse the attention planner's operand validation by planning a
     // same-shape launch over q (then k); nothing is enqueued from the plan
-    // except the pre-pass arguments assembled below.
-    ZdrawHipAttnExt sx;
+    // except the pre-pass arguments assembled below. Both operands are checked
+    // before the first launch, so a refused call leaves q untouched.
+    PrepArgs prs[2];
     for (int which = 0; which < 2; which++) {
         ZdrawAttnParams sp = *p;
         sp.heads = sp.kv_heads = which == 0 ? p->heads : p->kv_heads;
         sp.causal = 0;
         sp.valid = 0;
+        ZdrawHipAttnExt sx;
         standalone_ext(&sp, 0, 0, &sx);
         sx.qk_mode = x->qk_mode;
+        sx.k_site = ZDRAW_HIP_K_PREPASS; // typed norm weights are the pre-pass kernel's
         sx.eps = x->eps;
         sx.txt_rows = x->txt_rows;
         sx.rope_batch_rows = x->rope_batch_rows;
@@ -1020,23 +1150,20 @@ int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
         memcpy(sx.zimage_base, x->zimage_base, sizeof(sx.zimage_base));
         void* buf = which == 0 ? q : k;
         FusedPlan plan;
-        rc = plan_attention(qu->dev, buf, buf, buf, buf, &sp, &sx, ops, &plan);
+        ScratchSource none(qu->dev, /*dry=*/true);
+        rc = plan_attention(qu->dev, buf, buf, buf, buf, &sp, &sx, ops, &plan, &none, nw);
         if (rc != ZDRAW_HIP_OK) return rc;
-        PrepArgs pr;
-        memset(&pr, 0, sizeof(pr));
-        const AttnArgs& a = plan.args;
-        pr.x = a.q;
-        pr.y = a.o;
-        pr.x_bs = a.q_bs; pr.x_ts = a.q_ts; pr.x_hs = a.q_hs;
-        pr.y_bs = a.o_bs; pr.y_ts = a.o_ts; pr.y_hs = a.o_hs;
-        pr.tokens = a.tokens; pr.heads = a.heads; pr.batch = 1;
-        pr.mode = (int32_t)x->qk_mode;
+        // the plan's pre-pass describes the in-place form: same strides in and out, f32 out, no scale
+        PrepArgs pr = which == 0 ? plan.prep_q : plan.prep;
+        pr.y = const_cast<void*>(pr.x);
+        pr.y_bs = pr.x_bs; pr.y_ts = pr.x_ts; pr.y_hs = pr.x_hs;
+        pr.batch = 1;
         pr.out_dtype = kF32;
         pr.scale = 1.0f;
-        pr.qk = a.qk;
-        pr.w = which == 0 ? a.q_w : a.k_w;
-        pr.w_txt = which == 0 ? a.q_w_txt : a.k_w_txt;
-        hipError_t e = launch_qk_prepass(&pr, 1, kF32, qu->stream);
+        prs[which] = pr;
+    }
+    for (int which = 0; which < 2; which++) {
+        hipError_t e = launch_qk_prepass(&prs[which], 1, kF32, qu->stream);
         if (e != hipSuccess) {
             set_err("qk_norm_rope launch: %s", hipGetErrorString(e));
             return ZDRAW_HIP_ERR_HANDLE;
@@ -1047,6 +1174,43 @@ int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k,
     if (e != hipSuccess) return hip_fail(e, "qk_norm_rope wait");
     g_command++;
     return ZDRAW_HIP_OK;
+}
+} // namespace
+
+int zdraw_hip_run_qk_norm_rope_ext(void* queue, void* pipeline, void* q, void* k, const ZdrawAttnParams* p,
+                                   const ZdrawHipAttnExt* x, const ZdrawHipQkOperands* ops) {
+    return run_qk_norm_rope_impl(queue, pipeline, q, k, p, x, ops, nullptr);
+}
+
+// metal_c.zig:148-159, the dispatch behind mqk.run (metal/mqk.zig:20-58; kernel
+// metal/mqk_shader.zig:46-97, encode metal_api.m:6215-6265).
+int zdraw_hip_run_qk_norm_rope(void* queue, void* pipeline, void* q, void* k, void* q_weight, void* k_weight,
+                               void* pos, void* rope, const ZdrawQkNormParams* qp, size_t thread_count) {
+    (void)thread_count;
+    if (!qp) {
+        set_err("null params");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    ZdrawAttnParams p;
+    memset(&p, 0, sizeof(p));
+    p.tokens = qp->tokens;
+    p.heads = qp->heads;
+    p.kv_heads = qp->kv_heads;
+    p.head_dim = qp->head_dim;
+    ZdrawHipAttnExt x;
+    memset(&x, 0, sizeof(x));
+    x.qk_mode = ZDRAW_HIP_QK_ZIMAGE;
+    x.eps = qp->eps;
+    x.zimage_dims[0] = qp->dim0; x.zimage_dims[1] = qp->dim1; x.zimage_dims[2] = qp->dim2;
+    x.zimage_base[0] = qp->base0; x.zimage_base[1] = qp->base1; x.zimage_base[2] = qp->base2;
+    ZdrawHipQkOperands ops;
+    memset(&ops, 0, sizeof(ops));
+    ops.q_weight = q_weight;
+    ops.k_weight = k_weight;
+    ops.pos = pos;
+    ops.rope_pairs = rope;
+    const NormWeights nw{qp->q_dtype, qp->k_dtype, qp->q_offset, qp->k_offset};
+    return run_qk_norm_rope_impl(queue, pipeline, q, k, &p, &x, &ops, &nw);
 }
 
 // --------------------------------------------------------------------- gemm
@@ -1237,7 +1401,8 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
     ops.rope_pairs = w->rope;
     const NormWeights nw{p->qk.q_dtype, p->qk.k_dtype, p->qk.q_offset, p->qk.k_offset};
     FusedPlan plan;
-    int rc = plan_attention(b->queue->dev, bufs->q, bufs->k, bufs->v, bufs->mix, &at, &x, &ops, &plan, &nw);
+    ScratchSource slots(b->queue->dev);
+    int rc = plan_attention(b->queue->dev, bufs->q, bufs->k, bufs->v, bufs->mix, &at, &x, &ops, &plan, &slots, &nw);
     if (rc != ZDRAW_HIP_OK) return rc;
 
     ZdrawHipGemmExt gx;
@@ -1395,6 +1560,11 @@ void zdraw_hip_attention_tail_plan(uint64_t tiles, uint32_t cus, uint32_t key_bl
         attention_tail_plan((int64_t)tiles, (int)cus, (int)key_blocks, &t, &s);
     if (tail_tiles) *tail_tiles = (uint32_t)t;
     if (splits) *splits = (uint32_t)s;
+}
+
+int zdraw_hip_zimage_axis_lens(uint64_t table_bytes, const uint64_t* base, const uint32_t* dims, uint32_t* lens) {
+    if (!base || !dims || !lens) return ZDRAW_HIP_ERR_HANDLE;
+    return zimage_axis_lens(table_bytes, base, dims, lens) ? ZDRAW_HIP_OK : ZDRAW_HIP_INVALID;
 }
 
 size_t zdraw_hip_abi_sizeof(int which) {

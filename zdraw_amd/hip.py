@@ -1,4 +1,5 @@
-"""ctypes binding of the C ABI in include/zdraw_hip.h (libzdraw_hip.so)."""
+"""ctypes binding of the C ABI in include/zdraw_hip.h and of the measurement aids in
+include/zdraw_hip_measure.h (libzdraw_hip.so)."""
 from __future__ import annotations
 
 import ctypes as C
@@ -81,7 +82,7 @@ class ChainAttnParams(C.Structure):
 W_F16, W_BF16, W_F32 = 1, 2, 3     # weight dtype codes of GemmParams.dtype
 GEMM_EXACT, GEMM_HALF = 1, 2       # GemmParams.mode
 
-# every symbol include/zdraw_hip.h declares: name -> (restype, argtypes)
+# every symbol include/*.h declares: name -> (restype, argtypes)
 _vp, _sz, _u32, _u64, _int = C.c_void_p, C.c_size_t, C.c_uint32, C.c_uint64, C.c_int
 _AP, _AX, _QO = C.POINTER(AttnParams), C.POINTER(AttnExt), C.POINTER(QkOperands)
 _GP, _GX = C.POINTER(GemmParams), C.POINTER(GemmExt)
@@ -98,7 +99,7 @@ SYMBOLS = {
     "zdraw_hip_buffer_length": (_sz, [_vp]),
     "zdraw_hip_buffer_device_ptr": (_vp, [_vp]),
     "zdraw_hip_release_buffer": (None, [_vp]),
-    "zdraw_hip_compile": (_vp, [_vp, C.c_char_p, C.c_char_p, _sz]),
+    "zdraw_hip_compile": (_vp, [_vp, C.c_char_p, C.c_char_p, C.c_char_p, _sz]),
     "zdraw_hip_release_pipeline": (None, [_vp]),
     "zdraw_hip_pipeline_threads": (_sz, [_vp]),
     "zdraw_hip_run_attention": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _AP, _u32, _sz]),
@@ -108,7 +109,8 @@ SYMBOLS = {
     "zdraw_hip_batch_end": (_int, [_vp]),
     "zdraw_hip_run_attention_fused_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
     "zdraw_hip_run_attention_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
-    "zdraw_hip_run_qk_norm_rope": (_int, [_vp, _vp, _vp, _vp, _AP, _AX, _QO]),
+    "zdraw_hip_run_qk_norm_rope_ext": (_int, [_vp, _vp, _vp, _vp, _AP, _AX, _QO]),
+    "zdraw_hip_run_qk_norm_rope": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, C.POINTER(QkNormParams), _sz]),
     "zdraw_hip_attn_scratch": (_vp, [_vp, _int, _sz]),
     "zdraw_hip_metrics_reset": (None, []),
     "zdraw_hip_dispatch_count": (_u64, []),
@@ -127,7 +129,6 @@ SYMBOLS = {
     "zdraw_hip_run_gemm_group_ext_enc": (_int, [_vp, _vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_GP), C.c_uint32, _GX]),
     "zdraw_hip_run_chain_attn_enc": (_int, [_vp, C.POINTER(ChainAttnBuffers), C.POINTER(ChainAttnWeights),
                                             C.POINTER(ChainAttnParams)]),
-    "zdraw_hip_mfma_probe": (_int, [_int, _int, C.POINTER(C.c_double)]),
     "zdraw_hip_clock_probe": (None, [_int]),
     "zdraw_hip_clock_probe_read": (C.c_size_t, [C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_size_t]),
     "zdraw_hip_event_create": (_vp, []),
@@ -140,6 +141,7 @@ SYMBOLS = {
     "zdraw_hip_set_gemm_build": (None, [_int]),
     "zdraw_hip_attention_tail_plan": (None, [_u64, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "zdraw_hip_gemm_tail_plan": (None, [_u32, _u32, _u32, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "zdraw_hip_zimage_axis_lens": (_int, [_u64, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "zdraw_hip_abi_sizeof": (_sz, [_int]),
     "zdraw_hip_last_error": (C.c_char_p, []),
 }

@@ -42,6 +42,10 @@ void Buffer::deinit() {
 
 Error Context::init(Context* out) { return initKernel(Kernel::block, out); }
 
+// mattn.zig:69-118 hands zdraw_metal_compile the shader text of each kernel; the gfx950
+// kernels are compiled ahead of time, so there is no text to hand over.
+static const char* const kNoSource = "";
+
 Error Context::initKernel(Kernel kernel, Context* out) {
     Context c;
     c.device = zdraw_hip_create_device();
@@ -52,14 +56,14 @@ Error Context::initKernel(Kernel kernel, Context* out) {
         return Error::QueueFailed;
     }
     char err[256];
-    c.block_pipeline = zdraw_hip_compile(c.device, "attention_block_mfma", err, sizeof(err));
+    c.block_pipeline = zdraw_hip_compile(c.device, kNoSource, "attention_block_mfma", err, sizeof(err));
     if (!c.block_pipeline) {
         zdraw_hip_release_queue(c.queue);
         zdraw_hip_release_device(c.device);
         return Error::CompileFailed;
     }
-    c.qk_pipeline = zdraw_hip_compile(c.device, "qk_norm_rope", err, sizeof(err)); // optional, like mattn.zig:86
-    c.wide_pipeline = zdraw_hip_compile(c.device, "attention_wide_mfma", err, sizeof(err)); // optional, mattn.zig:83-85
+    c.qk_pipeline = zdraw_hip_compile(c.device, kNoSource, "qk_norm_rope", err, sizeof(err)); // optional, like mattn.zig:86
+    c.wide_pipeline = zdraw_hip_compile(c.device, kNoSource, "attention_wide_mfma", err, sizeof(err)); // optional, mattn.zig:83-85
     c.wide_threads = c.wide_pipeline ? zdraw_hip_pipeline_threads(c.wide_pipeline) : 0;
     c.kernel = kernel;
     c.threads = zdraw_hip_pipeline_threads(c.block_pipeline);

@@ -44,26 +44,23 @@ Error run(hattn::Context* ctx, void* q_h, void* k_h, const float* q_weight, cons
     hattn::Buffer rb = hattn::Buffer::fromBytes(ctx->device, rope.values, rope.count() * 2 * sizeof(float));
     Error result = Error::OutOfMemory;
     if (qw.handle && kw.handle && pb.handle && rb.handle) {
-        ZdrawAttnParams p{};
+        // mqk.zig:77-102 (makeParams): the weights are f32 views at offset 0 here
+        ZdrawQkNormParams p{};
         p.tokens = (uint32_t)cfg.tokens;
         p.heads = (uint32_t)cfg.heads;
         p.kv_heads = (uint32_t)cfg.kv_heads;
         p.head_dim = (uint32_t)cfg.head_dim;
-        ZdrawHipAttnExt x;
-        memset(&x, 0, sizeof(x));
-        x.qk_mode = ZDRAW_HIP_QK_ZIMAGE;
-        x.eps = cfg.norm_eps;
-        for (int a = 0; a < 3; a++) {
-            x.zimage_dims[a] = (uint32_t)rope.dims[a];
-            x.zimage_base[a] = rope.axisBase(a);
-        }
-        ZdrawHipQkOperands ops;
-        memset(&ops, 0, sizeof(ops));
-        ops.q_weight = qw.handle;
-        ops.k_weight = kw.handle;
-        ops.pos = pb.handle;
-        ops.rope_pairs = rb.handle;
-        result = fromCode(zdraw_hip_run_qk_norm_rope(ctx->queue, ctx->qk_pipeline, q_h, k_h, &p, &x, &ops));
+        p.q_dtype = p.k_dtype = ZDRAW_HIP_W_F32;
+        p.dim0 = (uint32_t)rope.dims[0];
+        p.dim1 = (uint32_t)rope.dims[1];
+        p.dim2 = (uint32_t)rope.dims[2];
+        p.eps = cfg.norm_eps;
+        p.q_offset = p.k_offset = 0;
+        p.base0 = rope.axisBase(0);
+        p.base1 = rope.axisBase(1);
+        p.base2 = rope.axisBase(2);
+        result = fromCode(zdraw_hip_run_qk_norm_rope(ctx->queue, ctx->qk_pipeline, q_h, k_h, qw.handle, kw.handle,
+                                                     pb.handle, rb.handle, &p, ctx->qk_threads));
     }
     qw.deinit();
     kw.deinit();
