@@ -714,12 +714,16 @@ def test_planted_keys_through_norm_and_rope_without_a_score_bound(ctx, k_site):
     rb = lambda a: host.bf16_bits_to_f32(host.f32_to_bf16_bits(a))
     qn = zo.klein_apply_rope(zo.klein_rms_norm_heads(rb(w.q[0]), wq), w.rope_cos, w.rope_sin)
     kn = zo.klein_apply_rope(zo.klein_rms_norm_heads(rb(w.k[0]), wk), w.rope_cos, w.rope_sin)
-    want = zo.attention_run(qn, kn, rb(w.v[0]), zo.Config(w.tokens, w.heads, w.heads, 128))
     scores = np.einsum("thd,shd->hts", qn, kn) / np.sqrt(128.0)
-    assert scores.max() - np.median(scores) > 30.0  # the case is about a wide spread of scores
-    # operands rounded to bf16 after norm and rope at such score magnitudes: the probabilities are
-    # sharp, and a row's output is one V row or a close mix; the bar is the bf16 bar
-    refimpl.check_close(got, want, "klein, wide scores, no bound")
+    assert scores.max() - np.median(scores) > 30.0 and scores.std() > 5.0  # the case is about a wide spread of scores
+    # With scores tens of nats apart the softmax is sharp, and the bf16 rounding of the prepared
+    # operands (a relative 2^-9 on every element) alone moves a probability by several percent:
+    # the oracle therefore takes the operands as the kernel's MFMAs see them, Q' = bf16(q' c) with
+    # c = log2(e) / sqrt(128) riding on it, K' = bf16(k'), and the usual bar applies
+    c = np.float32(1.4426950408889634 / np.sqrt(128.0))
+    want = zo.attention_run(rb(qn * c) / c, rb(kn), rb(w.v[0]), zo.Config(w.tokens, w.heads, w.heads, 128))
+    mx, mean = refimpl.check_close(got, want, "klein, wide scores, no bound")
+    say(f"  max abs {mx:.2e} mean abs {mean:.2e}")
     for b in bufs + wb + [o, cos, sin]:
         b.release()
 
