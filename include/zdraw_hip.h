@@ -184,6 +184,23 @@ int zdraw_hip_run_attention_fused(void* queue, void* q, void* k, void* v, void* 
                                   const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
                                   const ZdrawHipQkOperands* ops);
 
+/* The fused entry for callers that cannot allocate (no counterpart in the reference: it is
+ * for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc).
+ * Same arguments, results bit-identical to zdraw_hip_run_attention_fused_enc, but the prepared
+ * Q and K (the bf16 copy of an f32 V, the parts of key-split tiles) live in an array inside the
+ * library's device code instead of the grow-only slots: ZDRAW_HIP_NOALLOC_SCRATCH_BYTES per GPU,
+ * held until the process ends. A call that needs more (with bf16 operands:
+ * batch x heads x tokens x 512 bytes, plus 256 KiB per key-split tile part) returns 1 and
+ * enqueues nothing; the message says so. The call itself performs no device allocation and
+ * creates no events (it is left out of the attention trace and the clock probe). One array per
+ * GPU: calls that overlap on one GPU (two queues) race, calls on one queue are ordered. The
+ * first call that meets a norm-weight buffer reads its 128 weights back once (a blocking copy of
+ * 512 bytes) to form the score bound: make that call before a capture starts. */
+#define ZDRAW_HIP_NOALLOC_SCRATCH_BYTES (64u << 20)
+int zdraw_hip_run_attention_fused_noalloc_enc(void* batch, void* q, void* k, void* v, void* out,
+                                              const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                                              const ZdrawHipQkOperands* ops);
+
 /* ---- standalone QK-norm + rope --------------------------------------------
  * The general form (no counterpart declaration in the reference; it also serves the
  * in-place Klein krms_rope dispatches, klein/zflux2_resident.zig:1573-1579). In place on

@@ -23,6 +23,15 @@
 
 using namespace zdraw;
 
+// Scratch of zdraw_hip_run_attention_fused_noalloc_enc: the prepared Q and K (and the bf16 copy
+// of an f32 V, and the parts of key-split tiles) of ONE call. Every GPU the library runs on holds
+// its own copy of the array until the process ends; host code never uses the array's name as an
+// address, only what hipGetSymbolAddress returned for the device in question.
+constexpr size_t kNoallocScratchBytes = (size_t)ZDRAW_HIP_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kNoallocScratchBytes];
+constexpr int kMaxDevices = 16;
+static void* g_noalloc_scratch[kMaxDevices] = {};
+
 static_assert(sizeof(ZdrawAttnParams) == ZDRAW_HIP_ABI_ATTN_PARAMS_SIZE, "AttnParams ABI drift");
 static_assert(sizeof(ZdrawHipAttnExt) == ZDRAW_HIP_ABI_ATTN_EXT_SIZE, "AttnExt ABI drift");
 static_assert(sizeof(ZdrawHipQkOperands) == ZDRAW_HIP_ABI_QK_OPERANDS_SIZE, "QkOperands ABI drift");
@@ -566,8 +575,14 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     return ZDRAW_HIP_OK;
 }
 
-int enqueue(const FusedPlan& plan, hipStream_t stream) {
+// no_alloc: the call may not allocate: no clock probe buffer, no trace events, and the
+// kernels' one-time setup must already have happened (zdraw_hip_create_device does it).
+int enqueue(const FusedPlan& plan, hipStream_t stream, bool no_alloc = false) {
     if (!g_setup_done) {
+        if (no_alloc) {
+            set_err("attention kernels not set up: create the device first");
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
         hipError_t e = attention_setup();
         if (e != hipSuccess) {
             set_err("attention_setup: %s", hipGetErrorString(e));
@@ -585,7 +600,7 @@ int enqueue(const FusedPlan& plan, hipStream_t stream) {
         g_dispatch++;
     }
     AttnArgs args = plan.args;
-    if (g_clock_on) {
+    if (g_clock_on && !no_alloc) {
         if (!g_clock_buf && hipMalloc(&g_clock_buf, sizeof(unsigned long long) * 2 * kClockCap) != hipSuccess) g_clock_buf = nullptr;
         if (g_clock_buf) {
             args.clock_probe = g_clock_buf;
@@ -596,7 +611,7 @@ int enqueue(const FusedPlan& plan, hipStream_t stream) {
         }
     }
     TracePair tp{nullptr, nullptr};
-    if (g_trace && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
+    if (g_trace && !no_alloc && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
         (void)hipEventRecord(tp.a, stream);
     hipError_t e = launch_attention(args, plan.in_dtype, plan.k_mode, g_variant & 1, stream);
     if (e != hipSuccess) {
@@ -886,7 +901,28 @@ void* zdraw_hip_create_device(void) {
     // ZDRAW_ATTN_VARIANT picks the kernel build for a whole process (measurement aid)
     if (const char* v = getenv("ZDRAW_ATTN_VARIANT")) zdraw_hip_set_attention_variant(atoi(v));
     if (const char* v = getenv("ZDRAW_GEMM_BUILD")) gemm_set_build(atoi(v));
-    Device* d = new Device{0, prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256};
+    // One-time setup with the device current: the attention kernels' LDS limits (this also loads
+    // their code), and this device's address of the no-allocation entry's scratch array.
+    if (!g_setup_done) {
+        hipError_t e = attention_setup();
+        if (e != hipSuccess) {
+            set_err("attention_setup: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_setup_done = true;
+    }
+    const int ordinal = 0;
+    if (!g_noalloc_scratch[ordinal]) {
+        void* ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            set_err("hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_noalloc_scratch[ordinal] = ptr;
+    }
+    g_weight_max.reserve(256); // no host allocation when a call notes a weight buffer's maximum
+    Device* d = new Device{ordinal, prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256};
     return d;
 }
 
@@ -1098,6 +1134,30 @@ int zdraw_hip_run_attention_fused_enc(void* batch, void* q, void* k, void* v, vo
     int rc = plan_attention(b->queue->dev, q, k, v, out, params, ext, ops, &plan, &slots);
     if (rc != ZDRAW_HIP_OK) return rc;
     return enqueue(plan, b->queue->stream);
+}
+
+int zdraw_hip_run_attention_fused_noalloc_enc(void* batch, void* q, void* k, void* v, void* out,
+                                              const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                                              const ZdrawHipQkOperands* ops) {
+    Batch* b = static_cast<Batch*>(batch);
+    if (!b) {
+        set_err("null batch");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    Device* dev = b->queue->dev;
+    void* base = (dev->ordinal >= 0 && dev->ordinal < kMaxDevices) ? g_noalloc_scratch[dev->ordinal] : nullptr;
+    if (!base) {
+        set_err("no scratch array address for this device");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    // The array keeps the previous call's contents. Nothing in it has to start at zero: the
+    // pre-pass writes every prepared row before the attention kernel reads it, and the key-split
+    // parts write every row of every part before the merge reads them, in stream order.
+    ScratchSource span(dev, base, kNoallocScratchBytes);
+    FusedPlan plan;
+    int rc = plan_attention(dev, q, k, v, out, params, ext, ops, &plan, &span);
+    if (rc != ZDRAW_HIP_OK) return rc;
+    return enqueue(plan, b->queue->stream, /*no_alloc=*/true);
 }
 
 int zdraw_hip_run_attention_fused(void* queue, void* q, void* k, void* v, void* out,

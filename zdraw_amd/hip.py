@@ -14,6 +14,7 @@ K_ROWS, K_FLASH, K_BLOCK, K_WIDE = 0, 1, 2, 3
 F32, F16, BF16 = 0, 1, 2
 QK_NONE, QK_KLEIN, QK_ZIMAGE = 0, 1, 2
 K_IN_TILE_LOAD, K_PREPASS = 0, 1
+NOALLOC_SCRATCH_BYTES = 64 << 20  # ZDRAW_HIP_NOALLOC_SCRATCH_BYTES
 
 
 class AttnParams(C.Structure):
@@ -109,6 +110,7 @@ SYMBOLS = {
     "zdraw_hip_batch_end": (_int, [_vp]),
     "zdraw_hip_run_attention_fused_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
     "zdraw_hip_run_attention_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
+    "zdraw_hip_run_attention_fused_noalloc_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
     "zdraw_hip_run_qk_norm_rope_ext": (_int, [_vp, _vp, _vp, _vp, _AP, _AX, _QO]),
     "zdraw_hip_run_qk_norm_rope": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, C.POINTER(QkNormParams), _sz]),
     "zdraw_hip_attn_scratch": (_vp, [_vp, _int, _sz]),
