@@ -99,6 +99,85 @@ def spin_up(L, ctx, res, ms):
     return n
 
 
+def side_leg(L, ctx, w, *, bounded=True, spin_ms=300.0, warm=10, steps=100):
+    """A short measurement of one workload outside the driver-timed region: whole step
+    (pre-pass + attention, wall clock) and the attention kernel alone (its own HIP events)."""
+    from zdraw_amd import hip, workloads as wl
+
+    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_PREPASS, bounded=bounded)
+    spin_up(L, ctx, res, spin_ms)
+    timed_region(L, ctx, res, warm)
+    wall, kern_ms = timed_region(L, ctx, res, steps)
+    res.release()
+    return {"value": w.flops / (wall / steps) / 1e12, "kernel_tflops": w.flops / (kern_ms * 1e-3) / 1e12,
+            "kernel_frac": w.flops / (kern_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "ms_per_step": wall * 1e3 / steps,
+            "kernel_ms": kern_ms, "steps": steps}
+
+
+def attn_scale_main(args):
+    """`--workload attn_scale`: the reference's attention scaling measurement
+    (cmd/gemmbench.zig:631-678): plain attention through the standalone blocking entry on resident
+    f32 buffers, heads 30, head_dim 128, tokens 4224 / 8448 / 16896, best wall time of three calls
+    after one untimed call, as the reference takes it; the attention kernel's own device time
+    beside it. The line's `value` is the 16896-token figure."""
+    import numpy as np
+
+    from zdraw_amd import hip, host, workloads as wl
+
+    L = hip.lib()
+    ctx = host.Context.init()
+    heads = wl.ATTN_SCALE_HEADS
+    rows = {}
+    for tokens in wl.ATTN_SCALE_TOKENS:
+        x = wl.attn_scale_input(tokens)
+        qb, kb, vb = ctx.buffer(x), ctx.buffer(x), ctx.buffer(x)
+        ob = ctx.buffer(nbytes=x.nbytes)
+        p = hip.AttnParams(tokens, heads, heads, 128, 0, 0)
+
+        def call():
+            rc = L.zdraw_hip_run_attention(ctx.queue, ctx.block_pipeline, qb.handle, kb.handle, vb.handle, ob.handle,
+                                           C.byref(p), hip.K_BLOCK, 512)
+            if rc != 0:
+                raise RuntimeError(f"attention rc={rc}: {hip.last_error()}")
+
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < args.spinup_ms / 3:
+            call()
+        best = float("inf")
+        L.zdraw_hip_metrics_reset()
+        L.zdraw_hip_trace_attention(1)
+        for _ in range(max(args.steps, 3) if args.steps < 50 else 3):
+            t0 = time.perf_counter()
+            call()
+            best = min(best, time.perf_counter() - t0)
+        n = C.c_uint64(0)
+        kern_ns = L.zdraw_hip_trace_attention_ns(C.byref(n))
+        L.zdraw_hip_trace_attention(0)
+        out = ob.read(np.float32, x.shape)
+        if not np.isfinite(out).all():
+            raise RuntimeError("non-finite output")
+        flops = 4.0 * tokens * tokens * 128 * heads
+        rows[str(tokens)] = {"ms": best * 1e3, "tflops": flops / best / 1e12,
+                             "kernel_ms": kern_ns / 1e6 / max(n.value, 1),
+                             "kernel_tflops": flops / (kern_ns / 1e9 / max(n.value, 1)) / 1e12}
+        for b in (qb, kb, vb, ob):
+            b.release()
+    ctx.deinit()
+    last = rows[str(wl.ATTN_SCALE_TOKENS[-1])]
+    line = {
+        "metric": "attention TFLOP/s across token counts (heads 30, head_dim 128, resident f32 buffers, blocking call)",
+        "value": last["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": 3, "warmup": 1, "ms_per_step": last["ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "attn_scale: plain attention, H=30, D=128, S in 4224 / 8448 / 16896, f32 in and out "
+                               "(rounded to bf16 once, ahead of the kernel), best of three blocking calls",
+                   "tokens": rows},
+        "roofline": {"bound": "mfma", "achieved": last["kernel_tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": last["kernel_tflops"] / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "attn_fwd_kernel",
+                     "kernel_ms": last["kernel_ms"]},
+    }
+    print(json.dumps(line), flush=True)
+
+
 def gemm_main(args):
     """`--path gemm`: the projection GEMM C[m][n] = A[m][k] x W[n][k]^T on its own (bf16 operands
     and output, fp32 accumulation), by default the fused Q/K/V projection of a Klein 1024^2 block
@@ -362,12 +441,16 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--spinup-ms", type=float, default=1500.0,
                     help="untimed launches for this long before the warm-up steps (clock ramp from idle)")
-    ap.add_argument("--workload", default="klein_1024")
+    ap.add_argument("--workload", default="klein_1024",
+                    help="a benchmark shape (klein_1024, klein_512_x4, zimage_1024, klein_edit_ragged), or attn_scale: "
+                         "the reference's attention-scaling measurement (heads 30, 4224 / 8448 / 16896 tokens)")
     ap.add_argument("--k-site", choices=["tile", "prepass"], default=os.environ.get("ZDRAW_BENCH_K_SITE", "prepass"),
                     help="where K's norm+rope runs: inside the K-block load, or one pre-pass kernel per call")
     ap.add_argument("--variant", type=int, default=0, help="kernel shape: 0 = 8 waves, 1 = 4 waves x 2 workgroups")
     ap.add_argument("--dynamic-max", action="store_true", help="withhold the score bound (running-maximum softmax)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-side-legs", action="store_true",
+                    help="skip the short untimed-by-value legs (other softmax form, other benchmark shapes)")
     ap.add_argument("--cu-count", type=int, default=0,
                     help="confine the library's stream to this many compute units (0 = all): shows whether "
                          "the kernel's time follows the CU count or the board's power limit")
@@ -385,6 +468,8 @@ def main():
         return chain_main(args)
     if args.path == "wide":
         return wide_main(args)
+    if args.workload == "attn_scale":
+        return attn_scale_main(args)
 
     import numpy as np
 
@@ -433,16 +518,33 @@ def main():
     timed_region(L, ctx, res, 20)
     o_wall, _ = timed_region(L, ctx, res, 100)
 
+    res.release()
+    # Short legs outside the driver-timed region, for the record: the running-maximum softmax on
+    # the same workload (no score bound from the caller), and the other benchmark shapes.
+    side = {}
+    if not args.no_side_legs:
+        dyn = side_leg(L, ctx, w, bounded=args.dynamic_max)  # the softmax form the timed region did not run
+        side["dyn"] = dyn
+        for name in ("klein_512_x4", "zimage_1024", "klein_edit_ragged"):
+            if name == w.name:
+                continue
+            leg = side_leg(L, ctx, wl.by_name(name, seed=0), bounded=not args.dynamic_max,
+                           steps=50 if name == "klein_edit_ragged" else 100)
+            side[name] = {"value": leg["value"], "kernel_frac": leg["kernel_frac"], "ms_per_step": leg["ms_per_step"]}
+
     desc = (f"{w.name}: B={w.batch} H={w.heads} S={w.tokens} D=128 bf16, fused QK-RMSNorm + axial RoPE, "
             + ("no mask" if w.key_pad is None else "ragged key-padding mask"))
     flops = w.flops
     ms_per_step = wall * 1e3 / args.steps
     value = flops / (wall / args.steps) / 1e12
     achieved = flops / (kern_ms * 1e-3) / 1e12
-    traffic = None
+    # HBM bytes per launch come from profiler counters, which this run does not collect: the
+    # figure is the committed summary's (another run, another box) and is labelled as such
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", f"attn_fwd_{w.name}_traffic.json")
     if os.path.exists(tpath):
         traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        traffic_source = f"profiles/attn_fwd_{w.name}_traffic.json (static: rocprofv3 counters of an earlier run)"
     line = {
         "metric": "attn TFLOP/s + % of bf16 MFMA peak, Klein 1024^2 (H=24,S=4608,D=128)",
         "value": value,
@@ -465,6 +567,9 @@ def main():
             f"tflops_with_k_site_{other}": flops / (o_wall / 100) / 1e12,
             "untimed_spinup_launches": spun,
             **({"cu_count": args.cu_count} if args.cu_count > 0 else {}),
+            **({("tflops_bounded" if args.dynamic_max else "tflops_running_max"): side["dyn"]["value"],
+                ("kernel_frac_bounded" if args.dynamic_max else "kernel_frac_running_max"): side["dyn"]["kernel_frac"],
+                "other_workloads": {k: v for k, v in side.items() if k != "dyn"}} if side else {}),
         },
         "roofline": {
             "bound": "mfma",
@@ -473,12 +578,12 @@ def main():
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_BF16_TFLOPS,
             "traffic": traffic,
+            "traffic_source": traffic_source,
             "kernel": "attn_fwd_kernel",
             "kernel_ms": kern_ms,
             "shader_clock": clock,
         },
     }
-    res.release()
     ctx.deinit()
     if args.copy_calibration_mib:
         import torch

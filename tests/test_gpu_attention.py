@@ -957,3 +957,36 @@ def test_fused_zimage_entry_holds_device_positions_to_the_table(ctx):
     assert np.isfinite(outs[0]).all()
     assert np.array_equal(outs[0].view(np.uint32), outs[2].view(np.uint32))
     assert np.array_equal(outs[1].view(np.uint32), outs[3].view(np.uint32))
+
+
+# ------------------------------------ the reference's attention-scaling shapes
+def test_attention_scaling_shape_at_16896_tokens_sampled_rows(ctx):
+    # cmd/gemmbench.zig:631-678 times plain attention at heads 30 and 4224 / 8448 / 16896 tokens
+    # through the standalone entry on resident f32 buffers, q = k = v = one N(0, 0.01) array. The
+    # longest of them here, with sampled query tokens x all heads against the oracle (no CPU
+    # finishes all 16896), a byte-equal rerun and every row written.
+    L = hip.lib()
+    tokens, heads = wl.ATTN_SCALE_TOKENS[-1], wl.ATTN_SCALE_HEADS
+    say(f"attention scaling shape: {tokens} tokens x {heads} heads")
+    x = wl.attn_scale_input(tokens)
+    qb = ctx.buffer(x)
+    ob = ctx.buffer(nbytes=x.nbytes)
+    p = hip.AttnParams(tokens, heads, heads, 128, 0, 0)
+    outs = []
+    for _ in range(2):
+        rc = L.zdraw_hip_run_attention(ctx.queue, ctx.block_pipeline, qb.handle, qb.handle, qb.handle, ob.handle,
+                                       C.byref(p), hip.K_BLOCK, 512)
+        assert rc == 0, hip.last_error()
+        outs.append(ob.read(np.float32, x.shape))
+    qb.release()
+    ob.release()
+    got, again = outs
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    assert np.isfinite(got).all() and (np.abs(got).max(axis=-1) > 0).all()
+    rng = np.random.default_rng(2)
+    toks = sorted({0, 1, 255, 256, 8447, 8448, tokens - 257, tokens - 1} | set(rng.choice(tokens, 16, replace=False).tolist()))
+    want = zo.attention_token_list(x, x, x, zo.Config(tokens, heads, heads, 128), toks)
+    mx, mean = refimpl.check_close(got[toks], want, "attn_scale 16896")
+    say(f"  {len(toks)} query tokens x {heads} heads: max abs {mx:.2e} mean abs {mean:.2e}")
+    # the averages of 16896 values of size 0.1 are small: the bar in units of the output's own scale
+    assert mx <= 2e-2 * float(np.abs(want).max())

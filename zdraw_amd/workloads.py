@@ -124,6 +124,17 @@ def by_name(name: str, seed=0, small=False) -> Workload:
     raise KeyError(name)
 
 
+# The reference's attention-scaling measurement (cmd/gemmbench.zig:631-678): heads 30,
+# head_dim 128, these token counts; one N(0, 0.01) array serves as q, k and v.
+ATTN_SCALE_TOKENS = (4224, 8448, 16896)
+ATTN_SCALE_HEADS = 30
+
+
+def attn_scale_input(tokens, heads=ATTN_SCALE_HEADS, seed=0xA77) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    return rng.standard_normal((tokens, heads, HEAD_DIM), dtype=np.float32) * np.float32(0.1)
+
+
 NAMES = ("plumbing", "klein_1024", "klein_512_x4", "zimage_1024", "klein_edit_ragged")
 
 
