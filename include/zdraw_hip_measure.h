@@ -34,7 +34,10 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
 /* Which build of the attention kernel runs. Bit 0: 0 = 8 waves x 32 query rows per
  * workgroup, one workgroup per CU (default); 1 = 4 waves x 32 query rows, two workgroups
  * per CU. Bit 1: 2 = never split the tiles of a thinly filled last round along the keys
- * (by default they are). */
+ * (by default they are). Bit 2: 4 = the role-split build for prepared bf16 operands on the
+ * 8-wave shape (the two waves of a SIMD share 64 query rows: one forms the scores and the
+ * softmax, the other the product with V; a quarter less LDS traffic per MFMA, more cycles
+ * per key block: slower, kept for measurement). */
 void zdraw_hip_set_attention_variant(int variant);
 
 /* Which build multiplies 256 x 256 tiles of 16-bit activations. 1 = four waves, 128 x 128

@@ -935,6 +935,12 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     }
 }
 
+} // namespace fwd
+} // namespace zdraw
+namespace zdraw {
+namespace fwd {
+#include "attn_pair.hpp"
+
 constexpr int kMaxSplits = 16; // parts per key-split tile
 
 // Combines the parts of the key-split tiles: out[row] = sum_z O_z 2^(m_z - M) / sum_z l_z 2^(m_z - M),
@@ -994,6 +1000,23 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnArgs a, int b
 }
 
 // Whole tiles first, then (tail.splits > 1) the tiles of the last round in parts, then the merge.
+// The role-split build (attn_pair.hpp) runs prepared bf16 operands on the 8-wave shape when the
+// measurement knob asks for it; it reads a quarter less from LDS per MFMA but takes 30 % more
+// cycles per key block than the single-role kernel, which stays the default.
+static bool g_role_split = false;
+
+template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
+static void launch_kernel(const AttnArgs& a, unsigned grid, hipStream_t stream) {
+    if constexpr (std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && QB == 1 && NW == 8) {
+        if (g_role_split) {
+            pairk::attn_pair_kernel<MASKED, BOUNDED><<<dim3(grid), dim3(512), pairk::kLdsAlloc, stream>>>(a);
+            return;
+        }
+    }
+    attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
+        <<<dim3(grid), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
+}
+
 template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
 static hipError_t launch_one(const AttnArgs& a0, hipStream_t stream) {
     const int64_t nwg = (int64_t)a0.nqb * a0.heads * a0.batch;
@@ -1004,8 +1027,7 @@ static hipError_t launch_one(const AttnArgs& a0, hipStream_t stream) {
     a.splits = 1;
     const int64_t whole = nwg - tail;
     if (whole > 0) {
-        attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
-            <<<dim3((unsigned)whole), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
+        launch_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>(a, (unsigned)whole, stream);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -1013,8 +1035,7 @@ static hipError_t launch_one(const AttnArgs& a0, hipStream_t stream) {
         a.tile_base = (int32_t)whole;
         a.splits = a0.splits;
         a.clock_probe = nullptr;
-        attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
-            <<<dim3((unsigned)(tail * a0.splits)), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
+        launch_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>(a, (unsigned)(tail * a0.splits), stream);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         const int rows = tail * NW * 32 * QB;
@@ -1108,7 +1129,8 @@ int attention_key_block() { return fwd::KB; }
 int attention_max_tokens() { return fwd::MAX_BLOCKS * fwd::KB; }
 
 hipError_t launch_attention(const AttnArgs& a, int in_dtype, int k_mode, int shape, hipStream_t stream) {
-    switch (shape) {
+    fwd::g_role_split = (shape & 2) != 0;
+    switch (shape & 1) {
     case 0: return fwd::launch_shape<1, 8>(a, in_dtype, k_mode, stream);
     case 1: return fwd::launch_shape<1, 4>(a, in_dtype, k_mode, stream);
     default: return hipErrorInvalidValue;
@@ -1117,6 +1139,11 @@ hipError_t launch_attention(const AttnArgs& a, int in_dtype, int k_mode, int sha
 
 hipError_t attention_setup() {
     hipError_t e;
+#define ZD_RAISE_PAIR(M, B) \
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd::pairk::attn_pair_kernel<M, B>), \
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)fwd::pairk::kLdsAlloc)) != hipSuccess) return e;
+    ZD_RAISE_PAIR(false, false) ZD_RAISE_PAIR(false, true) ZD_RAISE_PAIR(true, false) ZD_RAISE_PAIR(true, true)
+#undef ZD_RAISE_PAIR
     if ((e = fwd::raise_shape<1, 8>()) != hipSuccess) return e;
     if ((e = fwd::raise_shape<1, 4>()) != hipSuccess) return e;
     return hipSuccess;

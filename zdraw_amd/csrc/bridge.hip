@@ -74,7 +74,7 @@ uint64_t g_dispatch = 0;
 uint64_t g_command = 0;
 uint64_t g_fallback = 0;
 uint64_t g_gpu_ns = 0;
-int g_variant = 0; // bit 0: kernel shape, 0 = 8 waves per workgroup, 1 = 4 waves (two workgroups per CU); bit 1: never split tail tiles
+int g_variant = 0; // bit 0: kernel shape, 0 = 8 waves per workgroup, 1 = 4 waves (two workgroups per CU); bit 1: never split tail tiles; bit 2: the role-split build where it applies (prepared bf16 operands, 8-wave shape)
 bool g_setup_done = false;
 bool g_gemm_setup_done = false;
 
@@ -613,7 +613,7 @@ int enqueue(const FusedPlan& plan, hipStream_t stream, bool no_alloc = false) {
     TracePair tp{nullptr, nullptr};
     if (g_trace && !no_alloc && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
         (void)hipEventRecord(tp.a, stream);
-    hipError_t e = launch_attention(args, plan.in_dtype, plan.k_mode, g_variant & 1, stream);
+    hipError_t e = launch_attention(args, plan.in_dtype, plan.k_mode, (g_variant & 1) | ((g_variant & 4) ? 2 : 0), stream);
     if (e != hipSuccess) {
         set_err("attention launch: %s", hipGetErrorString(e));
         return ZDRAW_HIP_ERR_HANDLE;
@@ -1596,7 +1596,7 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
     return m;
 }
 
-void zdraw_hip_set_attention_variant(int variant) { g_variant = variant & 3; }
+void zdraw_hip_set_attention_variant(int variant) { g_variant = variant & 7; }
 
 void zdraw_hip_set_gemm_build(int build) { gemm_set_build(build); }
 
