@@ -340,11 +340,15 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
                                  const ZdrawHipChainAttnWeights* weights,
                                  const ZdrawHipChainAttnParams* params);
 
-/* ---- library-owned scratch (metal_c.zig:321-325) -------------------------- */
-/* Grow-only, process-lifetime, filled at (re)allocation with 0x00 (0xFF when
- * ZDRAW_SCRATCH_POISON is set, metal_api.m:6147-6181). slot in [0, 7): 0-2 prepared
- * operands, 3-4 the parts of key-split attention tiles, 5 the parts of k-split GEMM tiles,
- * 6 a GEMM's f32 activations rounded to 16 bits. */
+/* ---- scratch slots (metal_c.zig:321-325) ----------------------------------
+ * The reference's process-lifetime, grow-only slots, for callers that keep their own
+ * intermediates in them: (re)allocated only to grow, filled at (re)allocation with 0x00
+ * (0xFF when ZDRAW_SCRATCH_POISON is set, metal_api.m:6147-6181). slot in [0, 7).
+ * The library's OWN scratch (prepared Q and K, V's bf16 copy, the parts of key-split
+ * attention tiles and of k-split GEMM tiles, rounded f32 activations) does not live here:
+ * every queue owns a private set of such slots, grown on the first call of a size on that
+ * queue (which waits for that queue's earlier work, then allocates) and freed with the queue,
+ * so work on two queues never shares scratch. */
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes);
 
 /* ---- counters and timing (metal_api.m:333-353, 420-433) ------------------- */

@@ -485,8 +485,8 @@ def test_queue_confined_to_fewer_compute_units_gives_the_same_bits(ctx, monkeypa
 
 def test_scratch_is_grow_only_and_filled(ctx):
     # metal_api.m:6147-6191: a slot is (re)allocated only to grow, and a new allocation is
-    # filled before anyone reads it. The library uses the slots itself (pre-passed Q and K,
-    # key-split parts), so the test grows slot 4 past whatever it holds now.
+    # filled before anyone reads it. (These are the caller's slots; the library's own scratch
+    # lives with its queues.)
     L = hip.lib()
     cur = L.zdraw_hip_attn_scratch(ctx.device, 4, 16)
     assert cur
@@ -503,6 +503,36 @@ def test_scratch_is_grow_only_and_filled(ctx):
     assert L.zdraw_hip_attn_scratch(ctx.device, 5, 16)      # the k-split GEMM tiles' parts
     assert L.zdraw_hip_attn_scratch(ctx.device, 6, 16)      # a GEMM's rounded f32 activations
     assert not L.zdraw_hip_attn_scratch(ctx.device, 7, 16)  # past the last slot
+
+
+def test_two_queues_do_not_share_scratch(ctx):
+    # The library's scratch (prepared Q and K, key-split parts) belongs to the queue a call runs
+    # on: two open batches on two queues of one device, their launches interleaved on the host,
+    # give the bits each workload gives alone.
+    L = hip.lib()
+    wa = wl.by_name("klein_512_x4", seed=41, small=True)
+    wb = wl.by_name("zimage_1024", seed=42, small=True)
+    ra = wl.Resident(ctx, wa, dtype=hip.BF16, k_site=hip.K_PREPASS)
+    rb = wl.Resident(ctx, wb, dtype=hip.BF16, k_site=hip.K_PREPASS)
+    alone_a, alone_b = ra.run(), rb.run()
+    q2 = L.zdraw_hip_create_queue(ctx.device)
+    assert q2
+    try:
+        for _ in range(3):
+            ra.o.write(np.zeros(ra.o.nbytes, np.uint8))
+            rb.o.write(np.zeros(rb.o.nbytes, np.uint8))
+            ba, bb = L.zdraw_hip_batch_begin(ctx.queue), L.zdraw_hip_batch_begin(q2)
+            assert ba and bb
+            for _ in range(4):
+                assert ra.launch(ba) == 0, hip.last_error()
+                assert rb.launch(bb) == 0, hip.last_error()
+            assert L.zdraw_hip_batch_end(bb) == 0 and L.zdraw_hip_batch_end(ba) == 0
+            assert np.array_equal(ra.read_output().view(np.uint32), alone_a.view(np.uint32))
+            assert np.array_equal(rb.read_output().view(np.uint32), alone_b.view(np.uint32))
+    finally:
+        L.zdraw_hip_release_queue(q2)
+    ra.release()
+    rb.release()
 
 
 # --------------------------------------------- standalone QK-norm + rope (mqk.run)

@@ -48,14 +48,19 @@ struct Device {
     int ordinal;
     int cus; // compute units: workgroup slots of the one-workgroup-per-CU kernels
 };
-struct Queue {
-    Device* dev;
-    hipStream_t stream;
-};
 struct Buffer {
     void* ptr;
     size_t len;
     bool owned;
+};
+constexpr int kScratchSlots = 7;
+struct Queue {
+    Device* dev;
+    hipStream_t stream;
+    // The library's own scratch (prepared operands, parts of split tiles, rounded activations):
+    // grow-only slots owned by the queue whose work uses them, so that two queues never share a
+    // byte of it; freed with the queue.
+    Buffer* scratch[kScratchSlots] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 };
 struct Pipeline {
     int kind; // 0 = attention_block_mfma, 1 = qk_norm_rope, 2 = gemm_half
@@ -176,17 +181,51 @@ bool need(const void* handle, size_t bytes) {
     return b && b->ptr && b->len >= bytes && ((uintptr_t)b->ptr % 16) == 0;
 }
 
-// Where a call's scratch comes from: the library's grow-only slots (zdraw_hip_attn_scratch),
+bool scratch_poisoned(int slot);
+
+// (Re)allocation of a grow-only scratch slot. `wait` drains whatever may still read the old
+// allocation before it is freed; the new one is filled (0x00, or 0xFF under
+// ZDRAW_SCRATCH_POISON) so that a read that precedes its write sees the same bytes on every
+// run (metal_api.m:6160-6181).
+template <typename Wait>
+Buffer* grow_slot(Buffer** slot_ptr, int slot, size_t bytes, Wait wait) {
+    Buffer* cur = *slot_ptr;
+    if (cur && cur->len >= bytes) return cur;
+    wait();
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        set_err("scratch hipMalloc(%zu) failed", bytes);
+        return nullptr;
+    }
+    (void)hipMemset(p, scratch_poisoned(slot) ? 0xFF : 0x00, bytes);
+    (void)hipDeviceSynchronize();
+    if (cur) {
+        (void)hipFree(cur->ptr);
+        cur->ptr = p;
+        cur->len = bytes;
+        return cur;
+    }
+    *slot_ptr = new Buffer{p, bytes, true};
+    return *slot_ptr;
+}
+
+// A queue's own slot: only work enqueued on this queue can be reading the old allocation.
+Buffer* queue_scratch(Queue* q, int slot, size_t bytes) {
+    if (!q || slot < 0 || slot >= kScratchSlots || bytes == 0) return nullptr;
+    return grow_slot(&q->scratch[slot], slot, bytes, [q] { (void)hipStreamSynchronize(q->stream); });
+}
+
+// Where a call's scratch comes from: the grow-only slots of the queue the call runs on,
 // or a caller-supplied span handed out piece by piece in 256-byte steps (the entry that
 // allocates nothing), or nowhere (a plan that is only validated).
 struct ScratchSource {
-    Device* dev;
+    Queue* queue;
     bool dry;
     char* span = nullptr; // bump allocation over [span, span + cap)
     size_t cap = 0, used = 0;
     bool over = false;    // the span was too small for what the call needs
-    ScratchSource(Device* d, bool dry_run = false) : dev(d), dry(dry_run) {}
-    ScratchSource(Device* d, void* base, size_t bytes) : dev(d), dry(false), span(static_cast<char*>(base)), cap(bytes) {}
+    ScratchSource(Queue* q, bool dry_run = false) : queue(q), dry(dry_run) {}
+    ScratchSource(Queue* q, void* base, size_t bytes) : queue(q), dry(false), span(static_cast<char*>(base)), cap(bytes) {}
     void* get(int slot, size_t bytes);
 };
 
@@ -665,8 +704,9 @@ bool g_wide_setup_done = false;
 // One wide head (metal/mattn.zig:261-275 widePick, :280-283 sdpaShape): f32 token-major
 // q, k, v, out [tokens][512] at byte offsets; rounds the operands into scratch slots 0-2,
 // then runs the wide kernel.
-int enqueue_wide(Device* dev, void* q, void* k, void* v, void* out, const ZdrawAttnParams* p, uint64_t in_off,
-                 uint64_t out_off, hipStream_t stream) {
+int enqueue_wide(Queue* queue, void* q, void* k, void* v, void* out, const ZdrawAttnParams* p, uint64_t in_off,
+                 uint64_t out_off) {
+    hipStream_t stream = queue->stream;
     if (p->tokens == 0) return unavailable("tokens == 0");
     if (p->heads != 1 || p->kv_heads != 1) return unavailable("the wide kernel runs one head");
     if (p->head_dim != (uint32_t)wide_head_dim()) return unavailable("the wide kernel runs head_dim 512");
@@ -684,7 +724,7 @@ int enqueue_wide(Device* dev, void* q, void* k, void* v, void* out, const ZdrawA
     }
     Buffer* sc[3];
     for (int i = 0; i < 3; i++) {
-        sc[i] = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, i, (size_t)n * 2));
+        sc[i] = queue_scratch(queue, i, (size_t)n * 2);
         if (!sc[i]) {
             set_err("scratch allocation failed");
             return ZDRAW_HIP_ERR_HANDLE;
@@ -743,7 +783,7 @@ int finish_blocking(Queue* qu, hipEvent_t start, hipEvent_t stop) {
     return ZDRAW_HIP_OK;
 }
 
-Buffer* g_scratch[7] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+Buffer* g_scratch[kScratchSlots] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 
 void* ScratchSource::get(int slot, size_t bytes) {
     if (dry) return reinterpret_cast<void*>(uintptr_t{256}); // never dereferenced: the plan is not launched
@@ -756,7 +796,7 @@ void* ScratchSource::get(int slot, size_t bytes) {
         used = at + bytes;
         return span + at;
     }
-    Buffer* b = static_cast<Buffer*>(zdraw_hip_attn_scratch(dev, slot, bytes));
+    Buffer* b = queue_scratch(queue, slot, bytes);
     return b ? b->ptr : nullptr;
 }
 
@@ -836,7 +876,7 @@ int enqueue_gemm_group(void* a, void* const* ws, void* const* cs, const uint64_t
     if (const size_t rb = gemm_round_bytes(g, (int)x->a_dtype)) {
         // f32 activations are rounded to the weight's type once, into scratch slot 6, and the
         // product then runs as for 16-bit activations
-        Buffer* a16 = static_cast<Buffer*>(zdraw_hip_attn_scratch(queue->dev, 6, rb));
+        Buffer* a16 = queue_scratch(queue, 6, rb);
         if (!a16) {
             set_err("scratch allocation failed");
             return ZDRAW_HIP_ERR_HANDLE;
@@ -850,7 +890,7 @@ int enqueue_gemm_group(void* a, void* const* ws, void* const* cs, const uint64_t
         int tail = 0, splits = 1;
         gemm_tail_plan(g, a_eff, queue->dev->cus, &tail, &splits);
         if (splits > 1) {
-            Buffer* part = static_cast<Buffer*>(zdraw_hip_attn_scratch(queue->dev, 5, gemm_part_bytes(tail, splits)));
+            Buffer* part = queue_scratch(queue, 5, gemm_part_bytes(tail, splits));
             if (!part) {
                 set_err("scratch allocation failed");
                 return ZDRAW_HIP_ERR_HANDLE;
@@ -944,19 +984,26 @@ void* zdraw_hip_create_queue(void* device) {
             set_err("hipExtStreamCreateWithCUMask failed");
             return nullptr;
         }
-        return new Queue{d, s};
+        { Queue* nq = new Queue; nq->dev = d; nq->stream = s; return nq; }
     }
     if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) {
         set_err("hipStreamCreate failed");
         return nullptr;
     }
-    return new Queue{d, s};
+    { Queue* nq = new Queue; nq->dev = d; nq->stream = s; return nq; }
 }
 
 void zdraw_hip_release_queue(void* queue) {
     Queue* q = static_cast<Queue*>(queue);
     if (!q) return;
     (void)hipStreamSynchronize(q->stream);
+    for (Buffer*& b : q->scratch) {
+        if (b) {
+            if (b->ptr) (void)hipFree(b->ptr);
+            delete b;
+            b = nullptr;
+        }
+    }
     (void)hipStreamDestroy(q->stream);
     delete q;
 }
@@ -1058,14 +1105,14 @@ int zdraw_hip_run_attention(void* queue, void* pipeline, void* q, void* k, void*
     FusedPlan plan;
     if (!wide) {
         standalone_ext(params, 0, 0, &x);
-        ScratchSource slots(qu->dev);
+        ScratchSource slots(qu);
         rc = plan_attention(qu->dev, q, k, v, output, params, &x, nullptr, &plan, &slots);
         if (rc != ZDRAW_HIP_OK) return rc;
     }
     hipEvent_t start, stop;
     if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return ZDRAW_HIP_ERR_HANDLE;
     (void)hipEventRecord(start, qu->stream);
-    rc = wide ? enqueue_wide(qu->dev, q, k, v, output, params, 0, 0, qu->stream) : enqueue(plan, qu->stream);
+    rc = wide ? enqueue_wide(qu, q, k, v, output, params, 0, 0) : enqueue(plan, qu->stream);
     if (rc == ZDRAW_HIP_OK) rc = finish_blocking(qu, start, stop);
     (void)hipEventDestroy(start);
     (void)hipEventDestroy(stop);
@@ -1096,11 +1143,11 @@ int zdraw_hip_run_attention_enc_off(void* batch, void* pipeline, void* q, void* 
     const bool wide = pipeline && static_cast<Pipeline*>(pipeline)->kind == 3;
     int rc = check_pipeline(pipeline, kernel, wide ? 3 : 0);
     if (rc != ZDRAW_HIP_OK) return rc;
-    if (wide) return enqueue_wide(b->queue->dev, q, k, v, o, params, in_off, out_off, b->queue->stream);
+    if (wide) return enqueue_wide(b->queue, q, k, v, o, params, in_off, out_off);
     ZdrawHipAttnExt x;
     standalone_ext(params, in_off, out_off, &x);
     FusedPlan plan;
-    ScratchSource slots(b->queue->dev);
+    ScratchSource slots(b->queue);
     rc = plan_attention(b->queue->dev, q, k, v, o, params, &x, nullptr, &plan, &slots);
     if (rc != ZDRAW_HIP_OK) return rc;
     return enqueue(plan, b->queue->stream);
@@ -1130,7 +1177,7 @@ int zdraw_hip_run_attention_fused_enc(void* batch, void* q, void* k, void* v, vo
         return ZDRAW_HIP_ERR_HANDLE;
     }
     FusedPlan plan;
-    ScratchSource slots(b->queue->dev);
+    ScratchSource slots(b->queue);
     int rc = plan_attention(b->queue->dev, q, k, v, out, params, ext, ops, &plan, &slots);
     if (rc != ZDRAW_HIP_OK) return rc;
     return enqueue(plan, b->queue->stream);
@@ -1153,7 +1200,7 @@ int zdraw_hip_run_attention_fused_noalloc_enc(void* batch, void* q, void* k, voi
     // The array keeps the previous call's contents. Nothing in it has to start at zero: the
     // pre-pass writes every prepared row before the attention kernel reads it, and the key-split
     // parts write every row of every part before the merge reads them, in stream order.
-    ScratchSource span(dev, base, kNoallocScratchBytes);
+    ScratchSource span(b->queue, base, kNoallocScratchBytes);
     FusedPlan plan;
     int rc = plan_attention(dev, q, k, v, out, params, ext, ops, &plan, &span);
     if (rc != ZDRAW_HIP_OK) return rc;
@@ -1210,7 +1257,7 @@ int run_qk_norm_rope_impl(void* queue, void* pipeline, void* q, void* k, const Z
         memcpy(sx.zimage_base, x->zimage_base, sizeof(sx.zimage_base));
         void* buf = which == 0 ? q : k;
         FusedPlan plan;
-        ScratchSource none(qu->dev, /*dry=*/true);
+        ScratchSource none(qu, /*dry=*/true);
         rc = plan_attention(qu->dev, buf, buf, buf, buf, &sp, &sx, ops, &plan, &none, nw);
         if (rc != ZDRAW_HIP_OK) return rc;
         // the plan's pre-pass describes the in-place form: same strides in and out, f32 out, no scale
@@ -1461,7 +1508,7 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
     ops.rope_pairs = w->rope;
     const NormWeights nw{p->qk.q_dtype, p->qk.k_dtype, p->qk.q_offset, p->qk.k_offset};
     FusedPlan plan;
-    ScratchSource slots(b->queue->dev);
+    ScratchSource slots(b->queue);
     int rc = plan_attention(b->queue->dev, bufs->q, bufs->k, bufs->v, bufs->mix, &at, &x, &ops, &plan, &slots, &nw);
     if (rc != ZDRAW_HIP_OK) return rc;
 
@@ -1490,29 +1537,10 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
 
 // ------------------------------------------------------------------ scratch
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes) {
-    if (!device || slot < 0 || slot >= 7 || bytes == 0) return nullptr;
-    Buffer* cur = g_scratch[slot];
-    if (cur && cur->len >= bytes) return cur;
-    // Grow: work already enqueued may still read the old allocation, so drain
-    // the device before it is freed.
-    (void)hipDeviceSynchronize();
-    void* p = nullptr;
-    if (hipMalloc(&p, bytes) != hipSuccess) {
-        set_err("scratch hipMalloc(%zu) failed", bytes);
-        return nullptr;
-    }
-    // Filled at (re)allocation so a read that precedes its write sees the same
-    // bytes on every run (metal_api.m:6160-6181).
-    (void)hipMemset(p, scratch_poisoned(slot) ? 0xFF : 0x00, bytes);
-    (void)hipDeviceSynchronize();
-    if (cur) {
-        (void)hipFree(cur->ptr);
-        cur->ptr = p;
-        cur->len = bytes;
-        return cur;
-    }
-    g_scratch[slot] = new Buffer{p, bytes, true};
-    return g_scratch[slot];
+    if (!device || slot < 0 || slot >= kScratchSlots || bytes == 0) return nullptr;
+    // The caller's slots (the reference's process-static set, metal_api.m:6147-6191). The
+    // library's own scratch lives with its queues, so nothing of the library reads these.
+    return grow_slot(&g_scratch[slot], slot, bytes, [] { (void)hipDeviceSynchronize(); });
 }
 
 // --------------------------------------------------------- counters, timing
