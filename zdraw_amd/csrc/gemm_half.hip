@@ -456,12 +456,12 @@ __global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArg
 // registers, 8 fragment reads per 16 MFMAs: a third fewer LDS bytes per MFMA than
 // the 8-wave builds). One wave per SIMD has no neighbour to hide its waits, so the
 // schedule leaves none: the fragments of the next 16-wide step are read under the
-// MFMAs of the current one, and the slab's one barrier sits after the THIRD of the
-// four steps: by then every fragment of the slab is in registers, so the barrier
-// both frees the slab's LDS stage for slab s + 2 (fetched at once, a whole slab
-// before it is needed) and makes slab s + 1 (fetched a slab ago) visible, whose
-// first fragments are then read under the MFMAs of the fourth step. Same 128-byte
-// swizzled rows and two 64 KB stages as the direct-to-LDS build above.
+// first MFMAs of the current one, and the slab's one barrier sits inside the THIRD of
+// the four steps, right after the slab's last fragments have reached registers: it
+// both frees the slab's LDS stage for slab s + 2 and makes slab s + 1 visible, whose
+// first fragments are read under the MFMAs of the fourth step. The loads of slab s + 2
+// follow the barrier one per two MFMAs. Same 128-byte swizzled rows and two 64 KB
+// stages as the direct-to-LDS build above.
 template <bool F16, typename TC>
 __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
     constexpr int TM = 4, TN = 4;
@@ -551,39 +551,50 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         if (r < 4) f.a[r] = *(lds_u32x4_t)(fa[kk] + stage_off + (unsigned)(r * 32 * (BK * 2)));
         else f.w[r - 4] = *(lds_u32x4_t)(fw[kk] + stage_off + (unsigned)((r - 4) * 32 * (BK * 2)));
     };
-    // 16 MFMAs on `cur`, the 8 reads of `nxt` spread under the first of them; fetch >= 0: one
-    // load of slab `fetch` per MFMA (a burst of 16 would hold the wave at the memory queue)
-    auto mfma_step = [&](const Frag& cur, Frag& nxt, unsigned nxt_stage_off, int nxt_kk, int fetch) __attribute__((always_inline)) {
+    // One 16-wide step: 16 MFMAs on `cur` with the 8 reads of `nxt` under the first of them.
+    // Step 2 carries the slab's barrier after its tenth MFMA: by then the last fragments of the
+    // slab are in registers (lgkmcnt(0)), so the barrier frees the slab's stage for slab s + 2
+    // and makes slab s + 1 visible (vmcnt(0): this wave's share of it has landed). The 16 loads
+    // of slab s + 2 are issued one per TWO MFMAs from there on (3 in the rest of step 2, 8 in
+    // step 3, 5 in step 0 of the next slab; the last has 33 MFMAs to land in). The CU's address
+    // unit takes 16 cycles per load and the four waves issue in the same phase: one load per
+    // MFMA from every wave held the waves at the memory queue for as long again as the step's
+    // MFMAs take (934 cycles for that step against 512 for the others).
+    auto mfma_step = [&](auto step_c, const Frag& cur, Frag& nxt, unsigned nxt_stage_off, int nxt_kk, int s) __attribute__((always_inline)) {
+        constexpr int STEP = decltype(step_c)::value;
 #pragma unroll
         for (int t = 0; t < 16; t++) {
-            if (fetch >= 0) fetch_one(fetch, t);
+            if (STEP == 0 && (t & 1) == 0 && t < 10) fetch_one(s + 1, 11 + (t >> 1));
+            if (STEP == 2 && (t & 1) == 0 && t >= 10) fetch_one(s + 2, (t - 10) >> 1);
+            if (STEP == 3 && (t & 1) == 0) fetch_one(s + 2, 3 + (t >> 1));
             if (t < 8) read_one(nxt, nxt_stage_off, nxt_kk, t);
             acc[t >> 2][t & 3] = mfma<F16>(cur.w[t & 3], cur.a[t >> 2], acc[t >> 2][t & 3]);
             __builtin_amdgcn_sched_barrier(0);
+            if (STEP == 2 && t == 9) {
+                __builtin_amdgcn_s_waitcnt(0x0070);
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     };
 
     fetch_slab(0);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
     __syncthreads();
-    fetch_slab(1);
+#pragma unroll
+    for (int i = 0; i < 11; i++) fetch_one(1, i); // the loop's first step sends the other five
     Frag f0, f1;
 #pragma unroll
     for (int r = 0; r < 8; r++) read_one(f0, 0u, 0, r);
     for (int s = 0; s < nslab; s++) {
         const unsigned so = (unsigned)(s & 1) * DMA_STAGE_BYTES;
         const unsigned so_next = (unsigned)((s + 1) & 1) * DMA_STAGE_BYTES;
-        mfma_step(f0, f1, so, 1, -1);
-        mfma_step(f1, f0, so, 2, -1);
-        mfma_step(f0, f1, so, 3, -1);
-        // every fragment of slab s is in registers (lgkmcnt(0)) and this wave's part of slab
-        // s + 1 has landed (vmcnt(0)): behind the barrier slab s's stage is free and slab s + 1
-        // is visible
-        __builtin_amdgcn_s_waitcnt(0x0070);
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        mfma_step(f1, f0, so_next, 0, s + 2);
+        mfma_step(std::integral_constant<int, 0>{}, f0, f1, so, 1, s);
+        mfma_step(std::integral_constant<int, 1>{}, f1, f0, so, 2, s);
+        mfma_step(std::integral_constant<int, 2>{}, f0, f1, so, 3, s);
+        mfma_step(std::integral_constant<int, 3>{}, f1, f0, so_next, 0, s);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
     if (g.splits > 1) {
