@@ -10,18 +10,24 @@
 // Shape of the computation on this machine:
 //   * a pre-pass rounds Q (times log2(e)/sqrt(512)), K and V to bf16 once, so the
 //     main kernel moves half the bytes and fetches blocks straight into LDS;
-//   * a workgroup of 8 waves owns 64 query rows: wave (g, s) owns query rows
-//     32 g .. 32 g + 31 and the 128-wide slice s of the 512 dims, as the
-//     reference's four simdgroups do. Every K/V byte is read once per workgroup;
-//   * per 32-key block a wave forms its partial S^T = K_s Q_s^T (8 MFMAs), the
-//     four partials of a query group are exchanged through LDS and summed in the
-//     written-out order ((p0 + p1) + p2) + p3 by each of the four waves, which
-//     then run the same online softmax redundantly (P must sit in every wave's
-//     registers for its own V slice anyway) and add V_s^T P^T to their slice of
-//     O^T (8 MFMAs). Scores are transposed (a lane owns one query), so P^T is
-//     the MFMA's B operand without an LDS round trip;
-//   * K/V blocks alternate between two LDS stages filled by buffer_load ... lds
-//     with the swizzled 256-byte-row layout of the head_dim-128 kernel;
+//   * a workgroup is four waves, one per SIMD (512 registers each), and owns 128 query
+//     rows and HALF of the 512 output dims; a wave owns 32 of the rows: its Q fragments
+//     (all 512 dims) and its O^T accumulators (256 dims) fill half the register file.
+//     Nothing is exchanged between waves and the softmax runs once per row and workgroup.
+//     The two workgroups of a query tile both form the full scores: 48 MFMAs per wave and
+//     32-key block where 32 would do, the price of an O tile that fits. (Owning all 512
+//     output dims needs 256 accumulation registers plus 128 for Q plus the pipeline's own:
+//     more than the compiler places without spilling into the loop.)
+//   * per block a wave forms S^T = K Q^T (32 MFMAs; scores transposed, so a lane owns one
+//     query and P^T is the next MFMA's B operand without an LDS round trip) with the online
+//     softmax of the previous block in their shadow, then adds V^T P^T to O^T (16 MFMAs);
+//   * K blocks (32 KB) and V half-blocks (16 KB) cycle through three LDS slots each, filled
+//     by buffer_load ... lds in the swizzled 256-byte-row layout of the head_dim-128 kernel.
+//     A block is requested two steps before it is used, and its 12 loads per wave are issued
+//     one per four MFMAs: the CU's address unit takes 16 cycles per load, and a burst from
+//     four waves at once holds them at the memory queue;
+//   * one barrier per block, placed after the 28th of the 32 S MFMAs, when the last K
+//     fragments are in registers: the V fragments of the product are read under the rest;
 //   * fixed block order and fixed summation order: bit-identical from run to run.
 #include "attn_device.hpp"
 
@@ -30,18 +36,22 @@ namespace zdraw {
 namespace wide {
 
 constexpr int WD = 512;           // head_dim
-constexpr int SL = 128;           // dims per slice
-constexpr int NSL = WD / SL;      // slices = waves per query group
+constexpr int SL = 128;           // dims per LDS tile ("slice")
+constexpr int NSL = WD / SL;
 constexpr int KB = 32;            // keys per block
-constexpr int NW = 8;
+constexpr int NW = 4;
 constexpr int NT = NW * 64;
-constexpr int BQ = 64;            // query rows per workgroup
-constexpr int TILE_BYTES = KB * SL * 2;            // one slice of a K (or V) block: 8 KB
-constexpr int RING_BYTES = NSL * TILE_BYTES;       // one K (or V) block, all slices: 32 KB
-constexpr int V_RING = 2 * RING_BYTES;             // two K slots, then two V slots
-constexpr int X_BYTES = 2 * NSL * 64 * 16 * 4;     // partial scores: [group][slice][4 x (lane x 16 B)]: 32 KB
-constexpr size_t kLdsBytes = (size_t)4 * RING_BYTES + X_BYTES;
+constexpr int BQ = 128;           // query rows per workgroup
+constexpr int HALF = WD / 2;      // output dims per workgroup
+constexpr int TILE_BYTES = KB * SL * 2;        // 8 KB
+constexpr int K_SLOT = NSL * TILE_BYTES;       // a K block: 32 KB
+constexpr int V_SLOT = (NSL / 2) * TILE_BYTES; // half the dims of a V block: 16 KB
+constexpr int NS = 3;                          // slots per ring
+constexpr int V_RING = NS * K_SLOT;
+constexpr size_t kLdsBytes = (size_t)NS * (K_SLOT + V_SLOT); // 144 KB
 constexpr float kTau = 8.0f;      // log2 headroom of the lazy softmax maximum
+constexpr int RA = 6;             // K fragments read ahead of their MFMA
+constexpr int VA = 3;             // V fragment pairs read ahead
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -64,169 +74,169 @@ __global__ void __launch_bounds__(256) wide_round_kernel(const WidePrepArgs p) {
     }
 }
 
-__global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
+template <int N> using IC = std::integral_constant<int, N>;
+
+__device__ __forceinline__ f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int j = 0; j < 16; j++) z[j] = 0.f;
+    return z;
+}
+
+__global__ void __launch_bounds__(NT, 1) attn_wide_kernel(const WideArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int l32 = lane & 31;
     const int h = lane >> 5;
-    const int grp = wave >> 2;  // query group
-    const int sl = wave & 3;    // dim slice
-    const int q0 = (int)blockIdx.x * BQ + 32 * grp;
+    const int dh = (int)blockIdx.x & 1;                      // which half of the output dims
+    const int q0 = ((int)blockIdx.x >> 1) * BQ + 32 * wave;  // this wave's query rows
     const int nblk = a.tokens / KB;
 
     const unsigned lds0 = lds_address(smem);
-    const unsigned xbase = lds0 + 4 * RING_BYTES;
 
-    // ---- Q fragments (B operand): query q0 + l32, dims 128 sl + 16 kk + 8 h .. +7
-    bf16x8 qf[8];
+    // ---- Q fragments (B operand of S^T = K Q^T): query q0 + l32, dims 16 kk + 8 h .. +7
+    bf16x8 qf[32];
     {
-        const bf16_t* qp = reinterpret_cast<const bf16_t*>(a.q) + (int64_t)(q0 + l32) * WD + SL * sl + 8 * h;
+        // rows past the end read the last row and are never stored
+        const bf16_t* qp = reinterpret_cast<const bf16_t*>(a.q) + (int64_t)min(q0 + l32, a.tokens - 1) * WD + 8 * h;
 #pragma unroll
-        for (int kk = 0; kk < 8; kk++) qf[kk] = *reinterpret_cast<const bf16x8*>(qp + 16 * kk);
+        for (int kk = 0; kk < 32; kk++) qf[kk] = *reinterpret_cast<const bf16x8*>(qp + 16 * kk);
     }
 
-    // ---- block fetch: wave w fills rows 16 (w >> 2) .. +15 of slice w & 3 of a K block or of a
-    // V block, four rows per instruction. The lane that fills chunk position p of row r
-    // fetches the chunk the swizzle places there: K chunk c of row r sits at c ^ (r & 15),
-    // V chunk c at c ^ ((r & 3) << 2). Positions past the last block re-fetch the last block
-    // into a slot nobody reads any more.
+    // ---- block fetch. K: wave w fills tile w (dims 128 w .. +127) of the block, four rows per
+    // instruction. V: wave w fills rows 16 (w >> 1) .. +15 of tile (w & 1) of this workgroup's
+    // half. The lane that fills chunk position p of row r fetches the chunk the swizzle places
+    // there: K chunk c of row r sits at c ^ (r & 15), V chunk c at c ^ ((r & 3) << 2).
     const unsigned span = (unsigned)a.tokens * (unsigned)(WD * 2);
     const u32x4 k_rsrc = make_rsrc_words(a.k, span);
     const u32x4 v_rsrc = make_rsrc_words(a.v, span);
-    unsigned fk_off[4], fv_off[4];
+    unsigned fk_off[4], fv_off[4]; // K rows 4 j + 16 take the same chunks 16 rows further on
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        const int row = 16 * grp + 4 * j + (lane >> 4);
+        const int row = 4 * j + (lane >> 4);
         const unsigned kc = (unsigned)((lane & 15) ^ (row & 15));
-        const unsigned vc = (unsigned)((lane & 15) ^ ((row & 3) << 2));
-        fk_off[j] = (unsigned)row * (WD * 2) + (unsigned)sl * (SL * 2) + kc * 16u;
-        fv_off[j] = (unsigned)row * (WD * 2) + (unsigned)sl * (SL * 2) + vc * 16u;
+        fk_off[j] = (unsigned)row * (WD * 2) + (unsigned)wave * (SL * 2) + kc * 16u;
     }
-    const unsigned fetch_lds = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)sl * TILE_BYTES + (unsigned)(16 * grp) * (SL * 2));
-    auto fetch_k = [&](int blk, int slot) __attribute__((always_inline)) {
-        const unsigned uo = (unsigned)(blk < nblk ? blk : nblk - 1) * (unsigned)(KB * WD * 2);
-        const unsigned base = fetch_lds + (unsigned)slot * RING_BYTES;
 #pragma unroll
-        for (int j = 0; j < 4; j++) load_to_lds_16(k_rsrc, base + (unsigned)(4 * j) * (SL * 2), fk_off[j], uo);
-    };
-    auto fetch_v = [&](int blk, int slot) __attribute__((always_inline)) {
-        const unsigned uo = (unsigned)(blk < nblk ? blk : nblk - 1) * (unsigned)(KB * WD * 2);
-        const unsigned base = fetch_lds + V_RING + (unsigned)slot * RING_BYTES;
-#pragma unroll
-        for (int j = 0; j < 4; j++) load_to_lds_16(v_rsrc, base + (unsigned)(4 * j) * (SL * 2), fv_off[j], uo);
-    };
-
-    // ---- fragment addresses in slot 0 of each ring (a slot adds a constant)
-    const int tr_row = (lane & 15) >> 2;
-    const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    unsigned kfo[8], vfo[4];
-#pragma unroll
-    for (int kk = 0; kk < 8; kk++)
-        kfo[kk] = lds0 + (unsigned)sl * TILE_BYTES + (unsigned)((l32 * SL + (((2 * kk + h) ^ (l32 & 15)) * 8)) * 2);
-#pragma unroll
-    for (int blk = 0; blk < 4; blk++)
-        vfo[blk] = lds0 + V_RING + (unsigned)sl * TILE_BYTES +
-                   (unsigned)(((4 * h + tr_row) * SL + ((blk ^ tr_row) * 32) + tr_col) * 2);
-    typedef const __attribute__((address_space(3))) bf16x8* lds_bf16x8_t;
-    typedef __attribute__((address_space(3))) s16x4* lds_s16x4_t;
-    typedef __attribute__((address_space(3))) f32x4* lds_f32x4_t;
-
-    // partial-score exchange: [group][slice][i < 4][lane] x 16 B
-    const unsigned x_mine = xbase + (unsigned)(((grp * NSL + sl) * 4) * 64 + lane) * 16u;
-    const unsigned x_group = xbase + (unsigned)((grp * NSL * 4) * 64 + lane) * 16u;
-    auto x_write = [&](const f32x16& sp) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            *(lds_f32x4_t)(x_mine + (unsigned)(i * 64 * 16)) = f32x4{sp[4 * i], sp[4 * i + 1], sp[4 * i + 2], sp[4 * i + 3]};
-    };
-    // full scores: ((p0 + p1) + p2) + p3, the same in each of the group's four waves
-    auto x_sum = [&](f32x16& sv) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            f32x4 t = *(lds_f32x4_t)(x_group + (unsigned)((0 * 4 + i) * 64 * 16));
-#pragma unroll
-            for (int s = 1; s < NSL; s++) {
-                const f32x4 u = *(lds_f32x4_t)(x_group + (unsigned)((s * 4 + i) * 64 * 16));
-                t += u;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) sv[4 * i + j] = t[j];
+    for (int j = 0; j < 4; j++) {
+        const int row = 16 * (wave >> 1) + 4 * j + (lane >> 4);
+        const unsigned vc = (unsigned)((lane & 15) ^ ((row & 3) << 2));
+        fv_off[j] = (unsigned)row * (WD * 2) + (unsigned)(2 * dh + (wave & 1)) * (SL * 2) + vc * 16u;
+    }
+    const unsigned fetch_k_lds = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)wave * TILE_BYTES);
+    const unsigned fetch_v_lds = __builtin_amdgcn_readfirstlane(lds0 + V_RING + (unsigned)(wave & 1) * TILE_BYTES + (unsigned)(16 * (wave >> 1)) * (SL * 2));
+    // the i-th (i < 12) load of the group that brings K block kb into K slot ks and V block vb into V slot vs
+    auto fetch_one = [&](int kb, int ks, int vb, int vs, int i) __attribute__((always_inline)) {
+        if (i < 8) {
+            const unsigned uo = (unsigned)(kb < nblk ? kb : nblk - 1) * (unsigned)(KB * WD * 2) + (unsigned)(i >> 2) * (16 * WD * 2);
+            load_to_lds_16(k_rsrc, fetch_k_lds + (unsigned)ks * K_SLOT + (unsigned)(4 * i) * (SL * 2), fk_off[i & 3], uo);
+        } else {
+            const unsigned uo = (unsigned)(vb < nblk ? vb : nblk - 1) * (unsigned)(KB * WD * 2);
+            load_to_lds_16(v_rsrc, fetch_v_lds + (unsigned)vs * V_SLOT + (unsigned)(4 * (i - 8)) * (SL * 2), fv_off[i - 8], uo);
         }
     };
 
-    f32x16 oacc[4]; // O^T slice: lane = query l32, dims 128 sl + 32 blk + 8 i + 4 h + j
+    // ---- fragment addresses in slot 0 (a tile and a slot add constants)
+    const int tr_row = (lane & 15) >> 2;
+    const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    // (pointers, so that the constant parts of an address go into the instruction's offset field)
+    typedef __attribute__((address_space(3))) unsigned char* lds_byte_t;
+    typedef const __attribute__((address_space(3))) bf16x8* lds_bf16x8_t;
+    typedef __attribute__((address_space(3))) s16x4* lds_s16x4_t;
+    const lds_byte_t lds_base = (lds_byte_t)smem;
+    lds_byte_t kfo[8], vfo[4];
+#pragma unroll
+    for (int kk = 0; kk < 8; kk++) kfo[kk] = lds_base + ((l32 * SL + (((2 * kk + h) ^ (l32 & 15)) * 8)) * 2);
 #pragma unroll
     for (int blk = 0; blk < 4; blk++)
+        vfo[blk] = lds_base + V_RING + (((4 * h + tr_row) * SL + ((blk ^ tr_row) * 32) + tr_col) * 2);
+    auto k_read = [&](int slot, int kk) __attribute__((always_inline)) {
+        return *(lds_bf16x8_t)(kfo[kk & 7] + (slot * K_SLOT + (kk >> 3) * TILE_BYTES));
+    };
+
+    f32x16 oacc[8]; // O^T: lane = query l32, dims 256 dh + 32 blk + 8 i + 4 h + j
+#pragma unroll
+    for (int blk = 0; blk < 8; blk++)
 #pragma unroll
         for (int j = 0; j < 16; j++) oacc[blk][j] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
-    // ---- prologue: K(0), K(1), V(0) in; scores of block 0 exchanged; K(2), V(1) requested.
-    // K runs one block ahead of V: step b multiplies by K(b+1) and by V(b).
-    fetch_k(0, 0);
-    fetch_v(0, 0);
-    fetch_k(1, 1);
+    // ---- prologue: K(0..2), V(0..1) in; S(0); then K(3) requested
+#pragma unroll
+    for (int i = 0; i < 12; i++) fetch_one(0, 0, 0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 12; i++) fetch_one(1, 1, 1, 1, i);
+#pragma unroll
+    for (int i = 0; i < 8; i++) fetch_one(2, 2, 0, 0, i);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
     __syncthreads();
     f32x16 sv; // scores of the block the next step exponentiates: lane = query l32, element 4 i + j = key 8 i + 4 h + j
     {
-        f32x16 sp;
+        f32x16 s = zero16();
 #pragma unroll
-        for (int j = 0; j < 16; j++) sp[j] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < 8; kk++)
-            sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(lds_bf16x8_t)(kfo[kk]), qf[kk], sp, 0, 0, 0);
-        x_write(sp);
-        __syncthreads();
-        x_sum(sv);
-        __syncthreads();
+        for (int kk = 0; kk < 32; kk++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_read(0, kk), qf[kk], s, 0, 0, 0);
+        sv = s;
     }
-    fetch_k(2, 0);
-    fetch_v(1, 1);
+    __syncthreads(); // K(0) has no reader left
+#pragma unroll
+    for (int i = 0; i < 4; i++) fetch_one(3, 0, 0, 0, i); // the first step sends the other eight of this group
+    bf16x8 kf[RA + 1]; // ring of fragments in flight
+#pragma unroll
+    for (int kk = 0; kk < RA; kk++) kf[kk] = k_read(1, kk);
 
-    // One step: the MFMAs of S(b+1) = K(b+1) Q^T (this wave's slice) run with the softmax of
-    // block b in their shadow, then O += V(b)^T P(b)^T; the partial scores of block b+1 are
-    // published between the two, and collected after the barrier that also says "block
-    // b+2's K and block b+1's V have landed, K(b+1) and V(b) have no reader left".
-    for (int b = 0; b < nblk; b++) {
-        const unsigned kso = (unsigned)((b + 1) & 1) * RING_BYTES;
-        const unsigned vso = (unsigned)(b & 1) * RING_BYTES;
-        bf16x8 kf[8];
-        s16x4 vlo[8], vhi[8];
+    // The running maximum moved (rare after the first blocks): O^T *= alpha, in place in the
+    // accumulation file. Written out by hand: left to the compiler, the two versions of O that
+    // meet after the branch cost more registers than there are.
+    auto rescale = [&](float alpha) __attribute__((always_inline)) {
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // MFMA results are read next
 #pragma unroll
-        for (int kk = 0; kk < 8; kk++) kf[kk] = *(lds_bf16x8_t)(kfo[kk] + kso);
-        auto v_read = [&](int idx) __attribute__((always_inline)) {
-            const int kb = idx >> 2, blk = idx & 3;
-            const unsigned va = vfo[blk] + vso + (unsigned)(16 * kb) * (SL * 2);
-            vlo[idx] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)va);
-            vhi[idx] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(va + 8u * (SL * 2)));
-        };
-        f32x16 sp;
+        for (int blk = 0; blk < 8; blk++)
 #pragma unroll
-        for (int j = 0; j < 16; j++) sp[j] = 0.f;
-        float mloc = 0.f, mc = 0.f, alpha = 1.f, psum = 0.f;
+            for (int j = 0; j < 16; j++) {
+                float x = oacc[blk][j], t;
+                asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1" : "+a"(x), "=&v"(t) : "v"(alpha));
+                oacc[blk][j] = x;
+            }
+        asm volatile("s_nop 7" ::: "memory"); // and feed the next MFMAs
+    };
+
+    // One step b with K(b+1) in K slot KS = (b + 1) % 3 and V(b) in V slot VS = b % 3:
+    //   S phase: the 32 MFMAs of S(b+1) = K(b+1) Q^T with the softmax of block b in their shadow;
+    //   barrier: K(b+2) and V(b) have landed (requested two steps ago), K(b+1) and V(b-1) have no
+    //            reader left;
+    //   PV phase: O += V(b)^T P(b)^T (16 MFMAs), the first fragments of K(b+2) read under them.
+    // The 12 loads that bring K(b+4) and V(b+2) into the two freed slots follow the barrier, 4
+    // under the PV phase and 8 under the next S phase.
+    auto step = [&](auto ks_c, auto vs_c, int b) __attribute__((always_inline)) {
+        constexpr int KS = decltype(ks_c)::value;       // slot of K(b+1); K(b+2) is in (KS + 1) % 3
+        constexpr int VS = decltype(vs_c)::value;       // slot of V(b); V(b-1) was in (VS + 2) % 3
+        constexpr int KN = (KS + 1) % 3;
+        f32x16 s;
+        float mloc = 0.f, mc = 0.f, alpha = 1.f, psum = 0.f, e_even = 0.f;
         bool up = false;
         unsigned pc[8];
-        auto exp_pair = [&](int pr) __attribute__((always_inline)) {
-            f32x2 pp;
-            pp[0] = __builtin_amdgcn_exp2f(sv[2 * pr] - mc);
-            pp[1] = __builtin_amdgcn_exp2f(sv[2 * pr + 1] - mc);
-            psum += pp[0] + pp[1];
-            pc[pr] = __builtin_bit_cast(unsigned, __builtin_convertvector(pp, bf16x2));
+        s16x4 vlo[VA + 1], vhi[VA + 1];
+        // idx < 16: tile idx >> 3 of the half, key half (idx >> 2) & 1, 32-dim block idx & 3
+        auto v_read = [&](int idx) __attribute__((always_inline)) {
+            const lds_byte_t va = vfo[idx & 3] + (VS * V_SLOT + (idx >> 3) * TILE_BYTES + (16 * ((idx >> 2) & 1)) * (SL * 2));
+            vlo[idx % (VA + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)va);
+            vhi[idx % (VA + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(va + 8 * (SL * 2)));
         };
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int g = 0; g < 8; g++) {
-            sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[g], qf[g], sp, 0, 0, 0);
-            // softmax of block b in the exp2 domain (the scale rides on Q) with a lazy maximum:
-            // the reference point moves only when this block's maximum exceeds it by more than kTau
-            if (g == 0) {
+        for (int t = 0; t < 32; t++) {
+            // the previous barrier's group: K(b+3) into the slot K(b) left, V(b+1) into V(b-2)'s
+            if ((t & 3) == 0) fetch_one(b + 3, (KS + 2) % 3, b + 1, (VS + 1) % 3, 4 + (t >> 2));
+            if (t + RA < 32) kf[(t + RA) % (RA + 1)] = k_read(KS, t + RA);
+            if (t >= 28 && t - 28 < VA) v_read(t - 28);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[t % (RA + 1)], qf[t], t == 0 ? zero16() : s, 0, 0, 0);
+            // softmax of block b in the exp2 domain (the scale rides on Q) with a lazy maximum: the
+            // reference point moves only when this block's maximum exceeds it by more than kTau
+            if (t == 0) {
                 mloc = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-                v_read(0);
-                v_read(1);
-            } else if (g == 1) {
+            } else if (t == 1) {
                 mloc = fmaxf(mloc, fmaxf(fmaxf(fmaxf(sv[8], sv[9]), fmaxf(sv[10], sv[11])), fmaxf(fmaxf(sv[12], sv[13]), fmaxf(sv[14], sv[15]))));
                 const float mlc = pair_max(mloc);
                 up = mlc > m_run + kTau;
@@ -234,52 +244,63 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
                 mc = (m_new == -INFINITY) ? 0.f : m_new;
                 alpha = __builtin_amdgcn_exp2f(m_run - mc);
                 m_run = m_new;
-                v_read(2);
-                v_read(3);
-            } else if (g < 6) {
-                exp_pair(2 * (g - 2));
-                exp_pair(2 * (g - 2) + 1);
-                if (g < 4) {
-                    v_read(2 * g);
-                    v_read(2 * g + 1);
+            } else if (t >= 3 && t < 19) {
+                const int e = t - 3; // one exponential per MFMA
+                const float x = __builtin_amdgcn_exp2f(sv[e] - mc);
+                psum += x;
+                if (e & 1) {
+                    f32x2 pp = {e_even, x};
+                    pc[e >> 1] = __builtin_bit_cast(unsigned, __builtin_convertvector(pp, bf16x2));
+                } else {
+                    e_even = x;
                 }
-            } else if (g == 6) {
+            } else if (t == 19) {
                 l_run = l_run * alpha + psum;
-                if (__any(up)) {
-#pragma unroll
-                    for (int blk = 0; blk < 4; blk++)
-#pragma unroll
-                        for (int j = 0; j < 16; j++) oacc[blk][j] *= alpha;
-                }
+                if (__any(up)) rescale(alpha);
             }
             __builtin_amdgcn_sched_barrier(0);
+            if (t == 27) {
+                // every fragment of K(b+1) is in registers; K(b+2), V(b) have landed: everything but
+                // the 12 loads sent since the last barrier
+                __builtin_amdgcn_s_waitcnt(0x007C); // vmcnt(12) lgkmcnt(0)
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         const bf16x8 p0 = __builtin_bit_cast(bf16x8, u32x4{pc[0], pc[1], pc[2], pc[3]});
         const bf16x8 p1 = __builtin_bit_cast(bf16x8, u32x4{pc[4], pc[5], pc[6], pc[7]});
-        // O^T slice += V_s(b)^T . P^T; the transposing read delivers keys in P's order
 #pragma unroll
-        for (int idx = 0; idx < 8; idx++) {
-            const bf16x8 vf = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(vlo[idx], vhi[idx], 0, 1, 2, 3, 4, 5, 6, 7));
-            oacc[idx & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, idx < 4 ? p0 : p1, oacc[idx & 3], 0, 0, 0);
-            if (idx == 1) x_write(sp); // the S MFMAs have drained by now
+        for (int idx = 0; idx < 16; idx++) {
+            if ((idx & 3) == 1) fetch_one(b + 4, KS, b + 2, (VS + 2) % 3, idx >> 2);
+            if (idx + VA < 16) v_read(idx + VA);
+            if (idx >= 16 - RA) kf[(idx - (16 - RA)) % (RA + 1)] = k_read(KN, idx - (16 - RA));
+            const bf16x8 vf = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(vlo[idx % (VA + 1)], vhi[idx % (VA + 1)], 0, 1, 2, 3, 4, 5, 6, 7));
+            const int ob = (idx >> 3) * 4 + (idx & 3);
+            oacc[ob] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, ((idx >> 2) & 1) ? p1 : p0, oacc[ob], 0, 0, 0);
+            if (idx == 4) sv = s; // the S MFMAs have drained by now
             __builtin_amdgcn_sched_barrier(0);
         }
-        // every wave has seen its own part of K(b+2) and V(b+1) land (requested a step ago)
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        fetch_k(b + 3, (b + 1) & 1);
-        fetch_v(b + 2, b & 1);
-        x_sum(sv);
-        __syncthreads(); // the exchange area is rewritten in the next step
+    };
+
+    int b = 0;
+    for (; b + 2 < nblk; b += 3) {
+        step(IC<1>{}, IC<0>{}, b);
+        step(IC<2>{}, IC<1>{}, b + 1);
+        step(IC<0>{}, IC<2>{}, b + 2);
     }
+    if (b < nblk) step(IC<1>{}, IC<0>{}, b);
+    if (b + 1 < nblk) step(IC<2>{}, IC<1>{}, b + 1);
     __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
 
     // ---- epilogue: O = O^T / l
     const float l_tot = pair_sum(l_run);
     const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    float* op = a.o + (int64_t)(q0 + l32) * WD + SL * sl;
+    float* op = a.o + (int64_t)(q0 + l32) * WD + HALF * dh;
+    if (q0 + l32 >= a.tokens) return;
 #pragma unroll
-    for (int blk = 0; blk < 4; blk++)
+    for (int blk = 0; blk < 8; blk++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             f32x4 v;
@@ -292,7 +313,7 @@ __global__ void __launch_bounds__(NT, 2) attn_wide_kernel(const WideArgs a) {
 } // namespace wide
 
 int wide_head_dim() { return wide::WD; }
-int wide_block_rows() { return wide::BQ; }
+int wide_block_rows() { return 64; } // the reference's tokens % 64 == 0; a last tile may be half full
 
 hipError_t launch_wide_round(const WidePrepArgs& p, hipStream_t stream) {
     if (p.chunks <= 0) return hipErrorInvalidValue;
@@ -303,8 +324,8 @@ hipError_t launch_wide_round(const WidePrepArgs& p, hipStream_t stream) {
 }
 
 hipError_t launch_wide_attention(const WideArgs& a, hipStream_t stream) {
-    if (a.tokens <= 0 || a.tokens % wide::BQ != 0) return hipErrorInvalidValue;
-    wide::attn_wide_kernel<<<dim3((unsigned)(a.tokens / wide::BQ)), dim3(wide::NT), wide::kLdsBytes, stream>>>(a);
+    if (a.tokens <= 0 || a.tokens % wide_block_rows() != 0) return hipErrorInvalidValue;
+    wide::attn_wide_kernel<<<dim3((unsigned)((a.tokens + wide::BQ - 1) / wide::BQ) * 2u), dim3(wide::NT), wide::kLdsBytes, stream>>>(a);
     return hipGetLastError();
 }
 
