@@ -82,6 +82,27 @@ def test_wide_head_sharp_softmax_and_large_scores(ctx):
         assert np.abs(want[i, 0] - v[j, 0]).max() < 1e-3  # the planted key really takes the whole row
 
 
+def test_wide_head_reference_point_moves_several_times(ctx):
+    # 1152 tokens (nine query tiles, 36 key blocks): rows whose best key so far is overtaken
+    # three times, 8 to 11 in the score each time, so the accumulated O is rescaled in place
+    # with earlier contributions still in it (each planted key keeps e^-8 .. e^-11 of the
+    # weight of the next); rows in every wave of a tile and in both halves of the output dims
+    # are checked against the oracle like all others.
+    tokens = 1152
+    rng = np.random.default_rng(78)
+    q, k, v = draw(rng, tokens)
+    rows = (5, 37, 70, 127, 600, 1151)
+    for n, i in enumerate(rows):
+        unit = q[i, 0] / np.linalg.norm(q[i, 0]) * np.sqrt(512.0)
+        for level, j in ((0.45, 40 + n), (0.8, 500 + n), (1.3, 1100 + n)):  # scores about 10, 18, 29
+            k[j, 0] = level * unit
+    got = ctx.run(q, k, v, host.Config(tokens, 1, 1, 512)).reshape(tokens, 1, 512)
+    want = zo.attention_run(q, k, v, zo.Config(tokens, 1, 1, 512))
+    refimpl.check_close(got, want, "several moves of the reference point")
+    for n, i in enumerate(rows):
+        assert np.abs(want[i, 0] - v[1100 + n, 0]).max() < 1e-2  # the last planted key takes the row
+
+
 def test_wide_head_refusals_leave_nothing_enqueued(ctx):
     L = hip.lib()
     d0 = L.zdraw_hip_dispatch_count()
