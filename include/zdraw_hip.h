@@ -184,6 +184,14 @@ int zdraw_hip_run_attention_fused(void* queue, void* q, void* k, void* v, void* 
                                   const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
                                   const ZdrawHipQkOperands* ops);
 
+/* Sizes the queue's private scratch for a later zdraw_hip_run_attention_fused_enc with the same
+ * arguments (no counterpart in the reference, whose slots are sized by their first use too): the
+ * fused call then finds its scratch in place and neither waits for the queue nor allocates inside
+ * an open batch. Enqueues nothing; returns what the fused call would return for these arguments. */
+int zdraw_hip_reserve_attention_fused(void* queue, void* q, void* k, void* v, void* out,
+                                      const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
+                                      const ZdrawHipQkOperands* ops);
+
 /* The fused entry for callers that cannot allocate (no counterpart in the reference: it is
  * for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc).
  * Same arguments, results bit-identical to zdraw_hip_run_attention_fused_enc, but the prepared
@@ -347,8 +355,8 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
  * The library's OWN scratch (prepared Q and K, V's bf16 copy, the parts of key-split
  * attention tiles and of k-split GEMM tiles, rounded f32 activations) does not live here:
  * every queue owns a private set of such slots, grown on the first call of a size on that
- * queue (which waits for that queue's earlier work, then allocates) and freed with the queue,
- * so work on two queues never shares scratch. */
+ * queue (which waits for that queue's earlier work, then allocates; zdraw_hip_reserve_attention_fused
+ * does that ahead of time) and freed with the queue, so work on two queues never shares scratch. */
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes);
 
 /* ---- counters and timing (metal_api.m:333-353, 420-433) ------------------- */

@@ -535,6 +535,42 @@ def test_two_queues_do_not_share_scratch(ctx):
     rb.release()
 
 
+def test_reserved_scratch_leaves_the_fused_call_nothing_to_allocate(ctx):
+    # zdraw_hip_reserve_attention_fused sizes a queue's private scratch ahead of time: device
+    # memory in use grows at the reservation and not again at the call, and the call gives the
+    # bits it gives on a queue that sized its scratch by itself.
+    import torch
+    L = hip.lib()
+    w = wl.by_name("klein_512_x4", seed=43)  # full size: 75 MB of prepared Q and K, too much to come out of a cached chunk
+    r = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_PREPASS)
+    alone = r.run()
+    q2 = L.zdraw_hip_create_queue(ctx.device)
+    assert q2
+    try:
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        rc = L.zdraw_hip_reserve_attention_fused(q2, r.q.handle, r.k.handle, r.v.handle, r.o.handle, C.byref(r.params),
+                                                 C.byref(r.ext), C.byref(r.ops))
+        assert rc == 0, hip.last_error()
+        free1 = torch.cuda.mem_get_info()[0]
+        assert free0 - free1 >= 64 << 20
+        r.o.write(np.zeros(r.o.nbytes, np.uint8))
+        d0 = L.zdraw_hip_dispatch_count()
+        b = L.zdraw_hip_batch_begin(q2)
+        assert r.launch(b) == 0, hip.last_error()
+        assert L.zdraw_hip_batch_end(b) == 0
+        assert L.zdraw_hip_dispatch_count() > d0
+        assert torch.cuda.mem_get_info()[0] == free1
+        assert np.array_equal(r.read_output().view(np.uint32), alone.view(np.uint32))
+        # a call the fused entry would refuse is refused here too, and reserves nothing
+        bad = hip.AttnParams(w.tokens, w.heads, w.heads, 64, 0, 0)
+        assert L.zdraw_hip_reserve_attention_fused(q2, r.q.handle, r.k.handle, r.v.handle, r.o.handle, C.byref(bad),
+                                                   C.byref(r.ext), C.byref(r.ops)) != 0
+    finally:
+        L.zdraw_hip_release_queue(q2)
+    r.release()
+
+
 # --------------------------------------------- standalone QK-norm + rope (mqk.run)
 def test_qk_norm_rope_in_place_matches_oracle(ctx):
     rng = np.random.default_rng(9)

@@ -37,26 +37,13 @@ namespace zdraw {
 
 namespace fwd {
 
-// Schedule constants of the pipelined step. They can be overridden on the
-// compiler command line to measure alternatives; the defaults are the measured best.
-#ifndef ZDRAW_LDS_LOOKAHEAD
-#define ZDRAW_LDS_LOOKAHEAD 4 // slots between an LDS fragment read and the MFMA that consumes it
-#endif
-#ifndef ZDRAW_READ_BATCH
-#define ZDRAW_READ_BATCH 2    // slots whose fragment reads are issued together (one wait per batch)
-#endif
-#ifndef ZDRAW_MFMA_PRIO
-#define ZDRAW_MFMA_PRIO 1     // wave priority while an MFMA is issued, builds that stage blocks through registers (0 = leave it alone)
-#endif
-#ifndef ZDRAW_MFMA_PRIO_DIRECT
-#define ZDRAW_MFMA_PRIO_DIRECT 0 // the same for the direct-to-LDS build
-#endif
-#ifndef ZDRAW_DIRECT_LDS
-#define ZDRAW_DIRECT_LDS 1    // prepared bf16 K/V blocks go from global memory straight into LDS
-#endif
-#ifndef ZDRAW_STORE_SLOT
-#define ZDRAW_STORE_SLOT 1    // slot after which a step moves its staged block into the ring
-#endif
+// Schedule constants of the pipelined step (the measured best of what was tried).
+constexpr int kLdsLookahead = 4;   // slots between an LDS fragment read and the MFMA that consumes it
+constexpr int kReadBatch = 2;      // slots whose fragment reads are issued together (one wait per batch)
+constexpr int kMfmaPrio = 1;       // wave priority while an MFMA is issued, builds that stage blocks through registers (0 = leave it alone)
+constexpr int kMfmaPrioDirect = 0; // the same for the direct-to-LDS build
+constexpr bool kDirectLds = true;  // prepared bf16 K/V blocks go from global memory straight into LDS
+constexpr int kStoreSlot = 1;      // slot after which a step moves its staged block into the ring
 
 constexpr int KB = 32;            // keys per block
 constexpr int KPITCH = D + 8;     // 272 B rows: 16-lane b128 reads spread over all banks
@@ -127,19 +114,19 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // 16 bytes at base + 16 i, so rows are 256 bytes without padding and bank
     // conflicts are avoided by swizzling the 16-byte chunk position instead:
     // K chunk c of row r sits at c ^ (r & 15), V chunk c of row r at c ^ ((r & 3) << 2).
-    constexpr bool DMA = ZDRAW_DIRECT_LDS && std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && NW == 8 && QB == 1;
+    constexpr bool DMA = kDirectLds && std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && NW == 8 && QB == 1;
     constexpr int KSTAGE = DMA ? KB * D : KS_ELEMS; // elements per ring stage
     constexpr int VSTAGE = DMA ? KB * D : VS_ELEMS;
     // a block enters the ring AHEAD steps before S needs its K (direct loads: one more step, to land)
     constexpr int AHEAD = NST == 8 ? (DMA ? 5 : 4) : 2;
-    constexpr int LA = ZDRAW_LDS_LOOKAHEAD;   // slots between an LDS fragment read and its MFMA
-    constexpr int RB = ZDRAW_READ_BATCH;      // slots whose reads are issued together (divides 16 and LA)
+    constexpr int LA = kLdsLookahead;   // slots between an LDS fragment read and its MFMA
+    constexpr int RB = kReadBatch;      // slots whose reads are issued together (divides 16 and LA)
     // Wave priority while an MFMA is being issued. The register-staged builds gain from it (the
     // masked one loses 13 % without). The direct-to-LDS build runs 5 % fewer cycles per
     // workgroup without the two s_setprio per MFMA; the chip sits on its power limit, so the
     // clock gives part of that back and 2 % is left.
-    constexpr int MFMA_PRIO = DMA ? ZDRAW_MFMA_PRIO_DIRECT : ZDRAW_MFMA_PRIO;
-    constexpr int STORE_SLOT = ZDRAW_STORE_SLOT; // slot after which the ring store is issued
+    constexpr int MFMA_PRIO = DMA ? kMfmaPrioDirect : kMfmaPrio;
+    constexpr int STORE_SLOT = kStoreSlot; // slot after which the ring store is issued
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* const Ks = reinterpret_cast<bf16_t*>(smem);
     bf16_t* const Vs = Ks + NST * KSTAGE;

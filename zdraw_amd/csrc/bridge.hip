@@ -1183,6 +1183,20 @@ int zdraw_hip_run_attention_fused_enc(void* batch, void* q, void* k, void* v, vo
     return enqueue(plan, b->queue->stream);
 }
 
+int zdraw_hip_reserve_attention_fused(void* queue, void* q, void* k, void* v, void* out, const ZdrawAttnParams* params,
+                                      const ZdrawHipAttnExt* ext, const ZdrawHipQkOperands* ops) {
+    Queue* qu = static_cast<Queue*>(queue);
+    if (!qu) {
+        set_err("null queue");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
+    // planning grows the queue's scratch slots to what the call needs (and reads the norm
+    // weights back for the score bound); nothing is enqueued
+    FusedPlan plan;
+    ScratchSource slots(qu);
+    return plan_attention(qu->dev, q, k, v, out, params, ext, ops, &plan, &slots);
+}
+
 int zdraw_hip_run_attention_fused_noalloc_enc(void* batch, void* q, void* k, void* v, void* out,
                                               const ZdrawAttnParams* params, const ZdrawHipAttnExt* ext,
                                               const ZdrawHipQkOperands* ops) {

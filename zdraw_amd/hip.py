@@ -109,6 +109,7 @@ SYMBOLS = {
     "zdraw_hip_run_attention_enc_off": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _AP, _u32, _sz, _u64, _u64]),
     "zdraw_hip_batch_end": (_int, [_vp]),
     "zdraw_hip_run_attention_fused_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
+    "zdraw_hip_reserve_attention_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
     "zdraw_hip_run_attention_fused": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
     "zdraw_hip_run_attention_fused_noalloc_enc": (_int, [_vp, _vp, _vp, _vp, _vp, _AP, _AX, _QO]),
     "zdraw_hip_run_qk_norm_rope_ext": (_int, [_vp, _vp, _vp, _vp, _AP, _AX, _QO]),
