@@ -115,7 +115,9 @@ struct WideArgs {
     const void* v; // bf16 [tokens][512]
     float* o;      // f32 [tokens][512]
     int32_t tokens; // multiple of 64
-    int32_t pad0;
+    int32_t splits; // key ranges per query tile (wide_splits; 0 or 1: none); > 1 needs the two buffers below
+    float* part_o;  // f32 [splits][tokens][512]: unnormalised O of each key range
+    float* part_ml; // f32 [splits][tokens][2]: its reference point and row sum
 };
 // f32 -> bf16 rounding of the three operands (Q with its scale) in one launch.
 struct WidePrepArgs {
@@ -127,6 +129,10 @@ struct WidePrepArgs {
 };
 int wide_head_dim();
 int wide_block_rows();
+// Key ranges per query tile that fill a device of `cus` compute units (1: no split), and the
+// bytes of part_o followed by part_ml they need.
+int wide_splits(int tokens, int cus);
+size_t wide_part_bytes(int tokens, int splits);
 hipError_t launch_wide_round(const WidePrepArgs& args, hipStream_t stream);
 hipError_t launch_wide_attention(const WideArgs& args, hipStream_t stream);
 hipError_t wide_setup();

@@ -28,6 +28,9 @@
 //     four waves at once holds them at the memory queue;
 //   * one barrier per block, placed after the 28th of the 32 S MFMAs, when the last K
 //     fragments are in registers: the V fragments of the product are read under the rest;
+//   * a short sequence (4096 tokens give 64 workgroups) is cut into key ranges, one workgroup
+//     each, until the launch fills the CUs; a range leaves its unnormalised O and its
+//     (reference point, row sum) in scratch and wide_merge_kernel combines them in range order;
 //   * fixed block order and fixed summation order: bit-identical from run to run.
 #include "attn_device.hpp"
 
@@ -52,6 +55,7 @@ constexpr size_t kLdsBytes = (size_t)NS * (K_SLOT + V_SLOT); // 144 KB
 constexpr float kTau = 8.0f;      // log2 headroom of the lazy softmax maximum
 constexpr int RA = 6;             // K fragments read ahead of their MFMA
 constexpr int VA = 3;             // V fragment pairs read ahead
+constexpr int kMaxSplits = 8;     // key ranges per query tile
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -90,9 +94,15 @@ __global__ void __launch_bounds__(NT, 1) attn_wide_kernel(const WideArgs a) {
     const int wave = tid >> 6;
     const int l32 = lane & 31;
     const int h = lane >> 5;
-    const int dh = (int)blockIdx.x & 1;                      // which half of the output dims
-    const int q0 = ((int)blockIdx.x >> 1) * BQ + 32 * wave;  // this wave's query rows
-    const int nblk = a.tokens / KB;
+    // workgroup = (query tile, key range, half of the output dims); a.splits is a power of two
+    const int dh = (int)blockIdx.x & 1;
+    const int nsp = a.splits > 1 ? a.splits : 1;
+    const int lg = __builtin_ctz((unsigned)nsp); // (shifts: an integer division would run on the vector unit)
+    const int part = ((int)blockIdx.x >> 1) & (nsp - 1);
+    const int q0 = (((int)blockIdx.x >> 1) >> lg) * BQ + 32 * wave; // this wave's query rows
+    const int per = (a.tokens / KB + nsp - 1) >> lg;
+    const int blk0 = part * per;                                    // this range's first key block
+    const int nblk = max(min(a.tokens / KB - blk0, per), 1);        // and how many it has (the host gives every range some)
 
     const unsigned lds0 = lds_address(smem);
 
@@ -130,10 +140,11 @@ __global__ void __launch_bounds__(NT, 1) attn_wide_kernel(const WideArgs a) {
     // the i-th (i < 12) load of the group that brings K block kb into K slot ks and V block vb into V slot vs
     auto fetch_one = [&](int kb, int ks, int vb, int vs, int i) __attribute__((always_inline)) {
         if (i < 8) {
-            const unsigned uo = (unsigned)(kb < nblk ? kb : nblk - 1) * (unsigned)(KB * WD * 2) + (unsigned)(i >> 2) * (16 * WD * 2);
+            // (uniform, but the compiler may have formed it in a vector register)
+            const unsigned uo = __builtin_amdgcn_readfirstlane((unsigned)(blk0 + (kb < nblk ? kb : nblk - 1)) * (unsigned)(KB * WD * 2) + (unsigned)(i >> 2) * (16 * WD * 2));
             load_to_lds_16(k_rsrc, fetch_k_lds + (unsigned)ks * K_SLOT + (unsigned)(4 * i) * (SL * 2), fk_off[i & 3], uo);
         } else {
-            const unsigned uo = (unsigned)(vb < nblk ? vb : nblk - 1) * (unsigned)(KB * WD * 2);
+            const unsigned uo = __builtin_amdgcn_readfirstlane((unsigned)(blk0 + (vb < nblk ? vb : nblk - 1)) * (unsigned)(KB * WD * 2));
             load_to_lds_16(v_rsrc, fetch_v_lds + (unsigned)vs * V_SLOT + (unsigned)(4 * (i - 8)) * (SL * 2), fv_off[i - 8], uo);
         }
     };
@@ -294,11 +305,23 @@ __global__ void __launch_bounds__(NT, 1) attn_wide_kernel(const WideArgs a) {
     if (b + 1 < nblk) step(IC<2>{}, IC<1>{}, b + 1);
     __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
 
-    // ---- epilogue: O = O^T / l
+    // ---- epilogue: O = O^T / l, or the range's share as it stands
     const float l_tot = pair_sum(l_run);
+    if (q0 + l32 >= a.tokens) return;
+    if (nsp > 1) {
+        float* op = a.part_o + ((int64_t)part * a.tokens + (q0 + l32)) * WD + HALF * dh;
+#pragma unroll
+        for (int blk = 0; blk < 8; blk++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) =
+                    f32x4{oacc[blk][4 * i], oacc[blk][4 * i + 1], oacc[blk][4 * i + 2], oacc[blk][4 * i + 3]};
+        // both halves of the dims hold the same reference point and row sum; one of them writes
+        if (dh == 0 && h == 0) *reinterpret_cast<f32x2*>(a.part_ml + ((int64_t)part * a.tokens + (q0 + l32)) * 2) = f32x2{m_run, l_tot};
+        return;
+    }
     const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
     float* op = a.o + (int64_t)(q0 + l32) * WD + HALF * dh;
-    if (q0 + l32 >= a.tokens) return;
 #pragma unroll
     for (int blk = 0; blk < 8; blk++)
 #pragma unroll
@@ -308,6 +331,39 @@ __global__ void __launch_bounds__(NT, 1) attn_wide_kernel(const WideArgs a) {
             for (int j = 0; j < 4; j++) v[j] = oacc[blk][4 * i + j] * inv_l;
             *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
         }
+}
+
+// Combines the key ranges of a split launch, in range order: with reference points m_p and row
+// sums l_p, O = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p, m = max_p m_p. A thread owns four
+// dims of one row; every range's load is sent before the first is used.
+__global__ void __launch_bounds__(256) wide_merge_kernel(const WideArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; // (row, dim / 4)
+    const int64_t row = i / (WD / 4);
+    if (row >= a.tokens) return;
+    const int c4 = (int)(i - row * (WD / 4));
+    float m[kMaxSplits], l[kMaxSplits];
+    f32x4 o[kMaxSplits];
+    float mm = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < kMaxSplits; p++)
+        if (p < a.splits) {
+            const f32x2 ml = *reinterpret_cast<const f32x2*>(a.part_ml + ((int64_t)p * a.tokens + row) * 2);
+            m[p] = ml[0];
+            l[p] = ml[1];
+            o[p] = *reinterpret_cast<const f32x4*>(a.part_o + ((int64_t)p * a.tokens + row) * WD + 4 * c4);
+            mm = fmaxf(mm, m[p]);
+        }
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float lt = 0.f;
+#pragma unroll
+    for (int p = 0; p < kMaxSplits; p++)
+        if (p < a.splits) {
+            const float w = (m[p] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[p] - mm);
+            acc += o[p] * w;
+            lt += l[p] * w;
+        }
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    *reinterpret_cast<f32x4*>(a.o + row * WD + 4 * c4) = acc * inv;
 }
 
 } // namespace wide
@@ -323,9 +379,31 @@ hipError_t launch_wide_round(const WidePrepArgs& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Key ranges per query tile: doubled while the launch still fits the device's CUs once and
+// every range keeps at least eight key blocks. 16384 tokens fill 256 CUs unsplit; 4096 tokens
+// (the mid-block at 512 px) would leave three quarters of them idle.
+int wide_splits(int tokens, int cus) {
+    const int tiles = (tokens + wide::BQ - 1) / wide::BQ;
+    const int nblk = tokens / wide::KB;
+    int s = 1;
+    while (s < wide::kMaxSplits && tiles * 2 * (s * 2) <= cus && nblk / (s * 2) >= 8 && nblk % (s * 2) == 0) s *= 2;
+    return s;
+}
+size_t wide_part_bytes(int tokens, int splits) {
+    return splits > 1 ? (size_t)splits * (size_t)tokens * (wide::WD + 2) * sizeof(float) : 0;
+}
+
 hipError_t launch_wide_attention(const WideArgs& a, hipStream_t stream) {
     if (a.tokens <= 0 || a.tokens % wide_block_rows() != 0) return hipErrorInvalidValue;
-    wide::attn_wide_kernel<<<dim3((unsigned)((a.tokens + wide::BQ - 1) / wide::BQ) * 2u), dim3(wide::NT), wide::kLdsBytes, stream>>>(a);
+    const int nsp = a.splits > 1 ? a.splits : 1;
+    if (nsp > wide::kMaxSplits || (nsp & (nsp - 1)) != 0 || (a.tokens / wide::KB) % nsp != 0) return hipErrorInvalidValue;
+    if (nsp > 1 && (a.part_o == nullptr || a.part_ml == nullptr)) return hipErrorInvalidValue;
+    const unsigned tiles = (unsigned)((a.tokens + wide::BQ - 1) / wide::BQ);
+    wide::attn_wide_kernel<<<dim3(tiles * (unsigned)nsp * 2u), dim3(wide::NT), wide::kLdsBytes, stream>>>(a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || nsp == 1) return e;
+    const int64_t threads = (int64_t)a.tokens * (wide::WD / 4);
+    wide::wide_merge_kernel<<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream>>>(a);
     return hipGetLastError();
 }
 

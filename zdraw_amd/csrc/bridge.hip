@@ -757,6 +757,17 @@ int enqueue_wide(Queue* queue, void* q, void* k, void* v, void* out, const Zdraw
     a.q = sc[0]->ptr; a.k = sc[1]->ptr; a.v = sc[2]->ptr;
     a.o = reinterpret_cast<float*>(static_cast<char*>(bs[3]->ptr) + out_off);
     a.tokens = (int32_t)p->tokens;
+    a.splits = wide_splits(a.tokens, queue->dev->cus);
+    if (a.splits > 1) {
+        // a short sequence runs as key ranges whose shares go through scratch slot 3
+        Buffer* part = queue_scratch(queue, 3, wide_part_bytes(a.tokens, a.splits));
+        if (!part) {
+            set_err("scratch allocation failed");
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        a.part_o = static_cast<float*>(part->ptr);
+        a.part_ml = a.part_o + (size_t)a.splits * (size_t)a.tokens * (size_t)wide_head_dim();
+    }
     TracePair tp{nullptr, nullptr};
     if (g_trace && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
         (void)hipEventRecord(tp.a, stream);
