@@ -540,6 +540,27 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
             for (int i = 0; i < 4; i++) pin(vfo[i]);
         }
+#ifdef HACK16
+        auto mfma_half = [&](int slot, int part) __attribute__((always_inline)) {
+            if (slot & 1) {
+                const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
+                const bf16x8 vf =
+                    __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(vlo[idx], vhi[idx], 0, 1, 2, 3, 4, 5, 6, 7));
+                f32x16& c = oacc[0][blk];
+                const int q = 2 * kb + part;
+                f32x4 c0 = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+                c0 = part ? __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_prev[0][kb], vf, c0, 0, 0, 0) : __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_prev[0][kb], c0, 0, 0, 0);
+                for (int j = 0; j < 4; j++) c[4 * q + j] = c0[j];
+            } else {
+                const int st = slot >> 1;
+                f32x16& c = s_next[0];
+                const int q = 2 * (st & 1) + part;
+                f32x4 c0 = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+                c0 = part ? __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[0][st], kf[st], c0, 0, 0, 0) : __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[st], qf[0][st], c0, 0, 0, 0);
+                for (int j = 0; j < 4; j++) c[4 * q + j] = c0[j];
+            }
+        };
+#endif
         auto mfma_slot = [&](int slot) __attribute__((always_inline)) {
             if (MFMA_PRIO) __builtin_amdgcn_s_setprio(MFMA_PRIO);
             if (slot & 1) {
@@ -645,8 +666,28 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                     else if constexpr (XSTEP) frag_read(stage_of(2), stage_of(0), slot - 16);
                 }
             }
+#if !defined(HACK16)
             mfma_slot(g);
             valu_slice(g);
+#elif HACK16 == 1
+            mfma_half(g, 0);
+            mfma_half(g, 1);
+            valu_slice(g);
+#elif HACK16 == 2
+            mfma_half(g, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            valu_slice(g);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_half(g, 1);
+#elif HACK16 == 3
+            // the VALU work of an even slot is split over the even slot's second half and the odd slot's first half
+            mfma_half(g, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if ((g & 1) == 0) valu_slice(g);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_half(g, 1);
+            if (g & 1) valu_slice(g);
+#endif
             // ring: block b+AHEAD (in this register set since two steps ago) goes to its stage,
             // whose previous tenant's last reader (V, NST-AHEAD-1 steps back) is at least one
             // barrier behind; then the set starts loading block b+AHEAD+2

@@ -79,6 +79,24 @@ __device__ __forceinline__ f32x16 mfma(const u32x4& a, const u32x4& b, const f32
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// v_mfma_f32_16x16x32: a lane supplies 8 consecutive k (chunk lane / 16 of the 32) of row lane % 16
+// and receives, of the 16 x 16 result, row lane % 16 of the second operand against rows
+// 4 (lane / 16) .. + 3 of the first. Per FLOP it moves half the accumulator bytes of the 32 x 32
+// form through the register file, and at the board's power limit that is worth clock.
+// Written as assembly with the accumulator tied to the result: given the builtin, the compiler
+// picks the three-address form for these 64 four-register accumulators and then moves them
+// around the accumulation file inside the loop (several copies per MFMA). The compiler inserts
+// no hazard waits around assembly: the caller keeps dependent MFMAs apart (here 64 MFMAs) and
+// calls mfma16_drain() before anything else reads the results.
+template <bool F16>
+__device__ __forceinline__ void mfma16(const u32x4& a, const u32x4& b, f32x4& c) {
+    if constexpr (F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma16_drain() {
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+}
+
 // A wave's (32 TM) x (32 TN) block of C. The MFMAs take the W fragment as their first
 // operand, so a lane holds row row0 + 32 i + l32 of C and, in register 4 r + jj of tile
 // (i, j), column col0 + 32 j + 8 r + 4 h + jj: four consecutive columns per r, stored as
@@ -126,7 +144,6 @@ __device__ __forceinline__ void store_tile(const GemmArgs& g, void* c, const f32
 // Needs: every direct load of the workgroup has landed and a barrier has passed since the last
 // fragment read; 16-byte aligned rows of C.
 constexpr int epi_pitch(int tn) { return 64 * tn + 16; } // bytes per staged row: keeps 16-byte alignment, spreads the banks
-constexpr size_t kRingLdsBytes = 4 * (size_t)128 * epi_pitch(4); // four-wave build: >= its two 64 KB slab stages
 template <bool F16, typename TC, int TM, int TN>
 __device__ __forceinline__ void store_tile_lds(const GemmArgs& g, void* c, const f32x16 (&acc)[TM][TN], unsigned lds_wave, int row0, int col0, int lane) {
     static_assert(sizeof(TC) == 2, "16-bit C only");
@@ -175,6 +192,97 @@ __device__ __forceinline__ void store_tile_lds(const GemmArgs& g, void* c, const
 #pragma unroll
                 for (int e = 0; e < 8; e++)
                     if (col + e < g.n) dst[e] = (unsigned short)(v[q][e >> 1] >> (16 * (e & 1)));
+            }
+        }
+    }
+}
+
+// The four-wave build's block of C: 8 x 8 tiles of 16 x 16. The MFMAs take the W fragment as
+// their first operand, so a lane (c = lane % 16, q = lane / 16) holds row row0 + 16 i + c of C
+// and, in tile (i, j), columns col0 + 16 j + 4 q .. + 3: a store instruction covers 16 rows x 64
+// contiguous bytes of f32.
+template <bool F16, typename TC>
+__device__ __forceinline__ void store_tile16(const GemmArgs& g, void* c, const f32x4 (&acc)[8][8], int row0, int col0, int lane) {
+    const int c16 = lane & 15, q = lane >> 4;
+    const bool vec = (g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) % (4 * sizeof(TC))) == 0);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int row = row0 + 16 * i + c16;
+        if (row >= g.m) continue;
+        TC* const crow = reinterpret_cast<TC*>(c) + (int64_t)row * g.ldc;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int col = col0 + 16 * j + 4 * q;
+            const f32x4 v = acc[i][j];
+            if (vec && col + 4 <= g.n) {
+                if constexpr (std::is_same<TC, float>::value) *reinterpret_cast<f32x4*>(crow + col) = v;
+                else if constexpr (F16) *reinterpret_cast<u32x2*>(crow + col) = __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4));
+                else *reinterpret_cast<u32x2*>(crow + col) = __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if (col + e >= g.n) break;
+                    if constexpr (std::is_same<TC, float>::value) crow[col + e] = v[e];
+                    else if constexpr (F16) { const _Float16 x = (_Float16)v[e]; crow[col + e] = __builtin_bit_cast(unsigned short, x); }
+                    else { const bf16_t x = (bf16_t)v[e]; crow[col + e] = __builtin_bit_cast(unsigned short, x); }
+                }
+            }
+        }
+    }
+}
+
+// The same block for a 16-bit C, as whole 256-byte rows: the wave turns 32 rows at a time (two
+// rows of tiles) through 8 KB of LDS that are its own and lie behind the slab stages, so no
+// barrier is needed and a wave that finishes its last slab early stores while the others still
+// multiply. Staged rows are 256 bytes without padding; the 16-byte chunk c of row r sits at
+// c ^ (r & 15), which spreads both the 8-byte writes (16 rows x 2 halves per half wave) and the
+// row-wise reads over all banks. A wave's LDS operations complete in order, so the reads of one
+// pass see its writes and the next pass's writes follow its reads.
+// Needs 16-byte aligned rows of C.
+constexpr int kEpiWaveBytes = 32 * 256;
+template <bool F16, typename TC>
+__device__ __forceinline__ void store_tile_lds16(const GemmArgs& g, void* c, const f32x4 (&acc)[8][8], unsigned lds_wave, int row0, int col0, int lane) {
+    static_assert(sizeof(TC) == 2, "16-bit C only");
+    typedef __attribute__((address_space(3))) u32x2* lds_u32x2_t;
+    typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
+    const int c16 = lane & 15, q = lane >> 4;
+    // write: row 16 (i & 1) + c16, bytes 32 j + 8 q .. + 8 = chunk 2 j + q / 2, half q & 1
+    const unsigned wbase = lds_wave + (unsigned)(c16 * 256 + (q & 1) * 8);
+    const unsigned wsw = (unsigned)(c16 ^ (q >> 1)); // (2 j + q / 2) ^ c16 = (2 j) ^ (c16 ^ (q / 2))
+    // read: row 4 p + lane / 16 (p < 8), chunk lane % 16
+    const int rr = lane >> 4, ch = lane & 15;
+    const int col = col0 + 8 * ch;
+    const bool whole = col + 8 <= g.n;
+    unsigned short* const cbase = reinterpret_cast<unsigned short*>(c) + (int64_t)(row0 + rr) * g.ldc + col;
+#pragma unroll
+    for (int ip = 0; ip < 4; ip++) {
+#pragma unroll
+        for (int ii = 0; ii < 2; ii++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const f32x4 v = acc[2 * ip + ii][j];
+                u32x2 pk;
+                if constexpr (F16) pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4));
+                else pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
+                *(lds_u32x2_t)(wbase + (unsigned)(ii * 16 * 256) + (((unsigned)(2 * j) ^ wsw) * 16u)) = pk;
+            }
+        u32x4 v[8];
+#pragma unroll
+        for (int p2 = 0; p2 < 8; p2++) {
+            const int r = 4 * p2 + rr;
+            v[p2] = *(lds_u32x4_t)(lds_wave + (unsigned)(r * 256) + (unsigned)((ch ^ (r & 15)) * 16));
+        }
+#pragma unroll
+        for (int p2 = 0; p2 < 8; p2++) {
+            const int row = row0 + 32 * ip + 4 * p2 + rr;
+            if (row >= g.m) continue;
+            unsigned short* const dst = cbase + (int64_t)(32 * ip + 4 * p2) * g.ldc;
+            if (whole) {
+                *reinterpret_cast<u32x4*>(dst) = v[p2];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (col + e < g.n) dst[e] = (unsigned short)(v[p2][e >> 1] >> (16 * (e & 1)));
             }
         }
     }
@@ -452,25 +560,28 @@ __global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArg
 }
 
 // ---------------------------------------------------------------------------
-// Four-wave build: one wave per SIMD, each owning 128 x 128 of C (256 accumulation
-// registers, 8 fragment reads per 16 MFMAs: a third fewer LDS bytes per MFMA than
-// the 8-wave builds). One wave per SIMD has no neighbour to hide its waits, so the
-// schedule leaves none: the fragments of the next 16-wide step are read under the
-// first MFMAs of the current one, and the slab's one barrier sits inside the THIRD of
-// the four steps, right after the slab's last fragments have reached registers: it
-// both frees the slab's LDS stage for slab s + 2 and makes slab s + 1 visible, whose
-// first fragments are read under the MFMAs of the fourth step. The loads of slab s + 2
-// follow the barrier one per two MFMAs. Same 128-byte swizzled rows and two 64 KB
-// stages as the direct-to-LDS build above.
+// Four-wave build: one wave per SIMD, each owning 128 x 128 of C as 8 x 8 tiles of
+// v_mfma_f32_16x16x32 (256 accumulation registers; 16 fragment reads per 64 MFMAs, a third
+// fewer LDS bytes per MFMA than the 8-wave builds). One wave per SIMD has no neighbour to hide
+// its waits, so the schedule leaves none. A 64-wide slab is two 32-wide steps of 64 MFMAs; the
+// 16 fragments of the next step are read one per two MFMAs under the first half of the current
+// one. The slab's one barrier sits in its FIRST step, after the 40th MFMA, when the slab's last
+// fragments are in registers: it both frees the slab's LDS stage for slab s + 2 and makes slab
+// s + 1 visible, whose first fragments are read under the second step. The 16 loads of slab
+// s + 2 follow the barrier one per four MFMAs (the CU's address unit takes 16 cycles per 1 KB
+// load and the four waves issue in the same phase: 64 cycles per round of loads). The loop is
+// unrolled over the two stages, so every LDS address is a pointer plus a constant. Same
+// 128-byte swizzled rows and two 64 KB stages as the direct-to-LDS build above; behind them
+// 8 KB per wave for the epilogue of a 16-bit C.
+constexpr size_t kRingLdsBytes = 2 * (size_t)DMA_STAGE_BYTES + 4 * (size_t)kEpiWaveBytes; // 160 KB
 template <bool F16, typename TC>
 __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
-    constexpr int TM = 4, TN = 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int l32 = lane & 31;
-    const int h = lane >> 5;
+    const int c16 = lane & 15;
+    const int q4 = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
     // a tile of the split last round: workgroup = (tile, part), the part is a range of slabs
     int logical, part_id = 0;
@@ -527,51 +638,49 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         for (int i = 0; i < 16; i++) fetch_one(s, i);
     };
 
-    f32x16 acc[TM][TN];
+    f32x4 acc[8][8];
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < 8; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+        for (int j = 0; j < 8; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // fragment addresses in stage 0: row (.. + l32), logical chunk 2 kk + h (kk < 4)
-    const int sw = (l32 >> 1) & 7;
-    unsigned fa[4], fw[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; kk++) {
-        const unsigned pos = (unsigned)(((2 * kk + h) ^ sw) * 16);
-        fa[kk] = lds0 + (unsigned)((wm * 128 + l32) * (BK * 2)) + pos;
-        fw[kk] = lds0 + (unsigned)(BM * BK * 2 + (wn * 128 + l32) * (BK * 2)) + pos;
-    }
+    // fragment addresses: row (.. + c16), logical chunk 4 ks + q4 (ks < 2) at c ^ ((row >> 1) & 7);
+    // a tile row adds 16 rows = 2 KB. (Pointers, so that the constant parts go into the
+    // instruction's offset field; a stage is 64 KB, beyond that field: one pointer per stage.)
+    typedef const __attribute__((address_space(3))) unsigned char* lds_byte_t;
     typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
-    struct Frag { u32x4 a[TM], w[TN]; };
-    // the r-th of the 8 reads of a fragment set
-    auto read_one = [&](Frag& f, unsigned stage_off, int kk, int r) __attribute__((always_inline)) {
-        if (r < 4) f.a[r] = *(lds_u32x4_t)(fa[kk] + stage_off + (unsigned)(r * 32 * (BK * 2)));
-        else f.w[r - 4] = *(lds_u32x4_t)(fw[kk] + stage_off + (unsigned)((r - 4) * 32 * (BK * 2)));
-    };
-    // One 16-wide step: 16 MFMAs on `cur` with the 8 reads of `nxt` under the first of them.
-    // Step 2 carries the slab's barrier after its tenth MFMA: by then the last fragments of the
-    // slab are in registers (lgkmcnt(0)), so the barrier frees the slab's stage for slab s + 2
-    // and makes slab s + 1 visible (vmcnt(0): this wave's share of it has landed). The 16 loads
-    // of slab s + 2 are issued one per TWO MFMAs from there on (3 in the rest of step 2, 8 in
-    // step 3, 5 in step 0 of the next slab; the last has 33 MFMAs to land in). The CU's address
-    // unit takes 16 cycles per load and the four waves issue in the same phase: one load per
-    // MFMA from every wave held the waves at the memory queue for as long again as the step's
-    // MFMAs take (934 cycles for that step against 512 for the others).
-    auto mfma_step = [&](auto step_c, const Frag& cur, Frag& nxt, unsigned nxt_stage_off, int nxt_kk, int s) __attribute__((always_inline)) {
-        constexpr int STEP = decltype(step_c)::value;
+    const lds_byte_t lds_base = (lds_byte_t)smem;
+    const int sw = (c16 >> 1) & 7;
+    lds_byte_t fa[2][2], fw[2][2]; // [stage][ks]
 #pragma unroll
-        for (int t = 0; t < 16; t++) {
-            if (STEP == 0 && (t & 1) == 0 && t < 10) fetch_one(s + 1, 11 + (t >> 1));
-            if (STEP == 2 && (t & 1) == 0 && t >= 10) fetch_one(s + 2, (t - 10) >> 1);
-            if (STEP == 3 && (t & 1) == 0) fetch_one(s + 2, 3 + (t >> 1));
-            if (t < 8) read_one(nxt, nxt_stage_off, nxt_kk, t);
-            acc[t >> 2][t & 3] = mfma<F16>(cur.w[t & 3], cur.a[t >> 2], acc[t >> 2][t & 3]);
+    for (int st = 0; st < 2; st++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const int pos = ((4 * ks + q4) ^ sw) * 16;
+            fa[st][ks] = lds_base + (st * DMA_STAGE_BYTES + (wm * 128 + c16) * (BK * 2) + pos);
+            fw[st][ks] = lds_base + (st * DMA_STAGE_BYTES + BM * BK * 2 + (wn * 128 + c16) * (BK * 2) + pos);
+        }
+    struct Frag { u32x4 a[8], w[8]; };
+    // the r-th of the 16 reads of a fragment set
+    auto read_one = [&](Frag& f, int st, int ks, int r) __attribute__((always_inline)) {
+        if (r < 8) f.a[r] = *(lds_u32x4_t)(fa[st][ks] + r * 16 * (BK * 2));
+        else f.w[r - 8] = *(lds_u32x4_t)(fw[st][ks] + (r - 8) * 16 * (BK * 2));
+    };
+    // One 32-wide step: 64 MFMAs on `cur`, the 16 reads of `nxt` under the first 32 of them.
+    // FIRST (the slab's first step): the barrier after the 40th MFMA, then loads 0..5 of slab
+    // s + 2, one per four MFMAs; the second step sends loads 6..15.
+    auto mfma_step = [&](auto first_c, auto st_c, auto ks_c, const Frag& cur, Frag& nxt, int s) __attribute__((always_inline)) {
+        constexpr bool FIRST = decltype(first_c)::value;
+        constexpr int NST = decltype(st_c)::value, NKS = decltype(ks_c)::value; // where nxt is read from
+#pragma unroll
+        for (int t = 0; t < 64; t++) {
+            if (FIRST && t >= 40 && (t & 3) == 0) fetch_one(s + 2, (t - 40) >> 2);
+            if (!FIRST && (t & 3) == 1 && t < 40) fetch_one(s + 2, 6 + (t >> 2));
+            if ((t & 1) == 0 && t < 32) read_one(nxt, NST, NKS, t >> 1);
+            mfma16<F16>(cur.w[t & 7], cur.a[t >> 3], acc[t >> 3][t & 7]);
             __builtin_amdgcn_sched_barrier(0);
-            if (STEP == 2 && t == 9) {
-                __builtin_amdgcn_s_waitcnt(0x0070);
+            if (FIRST && t == 39) {
+                __builtin_amdgcn_s_waitcnt(0x0070); // vmcnt(0) lgkmcnt(0)
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
@@ -581,52 +690,54 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
     };
 
     fetch_slab(0);
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    fetch_slab(1);
+    __builtin_amdgcn_s_waitcnt(0x4F70); // vmcnt(16): slab 0 has landed
     __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 11; i++) fetch_one(1, i); // the loop's first step sends the other five
     Frag f0, f1;
 #pragma unroll
-    for (int r = 0; r < 8; r++) read_one(f0, 0u, 0, r);
-    for (int s = 0; s < nslab; s++) {
-        const unsigned so = (unsigned)(s & 1) * DMA_STAGE_BYTES;
-        const unsigned so_next = (unsigned)((s + 1) & 1) * DMA_STAGE_BYTES;
-        mfma_step(std::integral_constant<int, 0>{}, f0, f1, so, 1, s);
-        mfma_step(std::integral_constant<int, 1>{}, f1, f0, so, 2, s);
-        mfma_step(std::integral_constant<int, 2>{}, f0, f1, so, 3, s);
-        mfma_step(std::integral_constant<int, 3>{}, f1, f0, so_next, 0, s);
+    for (int r = 0; r < 16; r++) read_one(f0, 0, 0, r);
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    int s = 0;
+    for (; s + 1 < nslab; s += 2) {
+        mfma_step(std::true_type{}, I0{}, I1{}, f0, f1, s);
+        mfma_step(std::false_type{}, I1{}, I0{}, f1, f0, s);
+        mfma_step(std::true_type{}, I1{}, I1{}, f0, f1, s + 1);
+        mfma_step(std::false_type{}, I0{}, I0{}, f1, f0, s + 1);
+    }
+    if (s < nslab) {
+        mfma_step(std::true_type{}, I0{}, I1{}, f0, f1, s);
+        mfma_step(std::false_type{}, I1{}, I0{}, f1, f0, s);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
+    mfma16_drain();
     if (g.splits > 1) {
-        // partial tile in the accumulation layout: [tile][part][wave][i][j][r][lane] x 16 bytes,
+        // partial tile in the accumulation layout: [tile][part][wave][i][j][lane] x 16 bytes,
         // every store instruction 1 KB in a row; the merge kernel reads it the same way
         f32x4* dst = reinterpret_cast<f32x4*>(g.part) +
                      ((((int64_t)(logical - g.tile_base) * g.splits + part_id) * 4 + wave) * 64) * 64 + lane;
 #pragma unroll
-        for (int i = 0; i < TM; i++)
+        for (int i = 0; i < 8; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++)
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    dst[(i * 16 + j * 4 + r) * 64] = f32x4{acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2], acc[i][j][4 * r + 3]};
+            for (int j = 0; j < 8; j++) dst[(i * 8 + j) * 64] = acc[i][j];
         return;
     }
     if constexpr (sizeof(TC) == 2) {
         // uniform over the launch: rows of C start on 16 bytes
         if ((g.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(cp) % 16 == 0)) {
-            __syncthreads(); // every wave's loads have landed and its fragments are read: the ring is idle
-            store_tile_lds<F16, TC, TM, TN>(g, cp, acc, lds0 + (unsigned)wave * (128 * epi_pitch(TN)), m0 + wm * 128, n0 + wn * 128, lane);
+            store_tile_lds16<F16, TC>(g, cp, acc, lds0 + 2u * DMA_STAGE_BYTES + (unsigned)wave * kEpiWaveBytes, m0 + wm * 128, n0 + wn * 128, lane);
             return;
         }
     }
-    store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, l32, h);
+    store_tile16<F16, TC>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, lane);
 }
 
 // Adds the parts of the k-split tiles in part order and writes C. A workgroup takes the 32 x
 // 128 block (tile, wave, i) of the four-wave build's accumulation layout: its wave j owns the
-// tiles (i, j), a lane row 32 i + lane % 32 and, for r < 4, columns 32 j + 8 r + 4 (lane / 32)
-// .. + 4. Every part's load (4 x splits of 16 bytes per lane) is sent before the first is
-// used; the sums are turned through LDS so that C is stored as whole rows of the block.
+// 16 x 16 tiles (2 i + r / 2, 2 j + r % 2), r < 4; a lane holds row lane % 16 and columns
+// 4 (lane / 16) .. + 4 of each. Every part's load (4 x splits of 16 bytes per lane) is sent
+// before the first is used; the sums are turned through LDS so that C is stored as whole rows
+// of the block.
 constexpr int kMaxKSplits = 8;
 template <bool F16, typename TC>
 __global__ void __launch_bounds__(256) gemm_merge_kernel(const GemmArgs g) {
@@ -636,24 +747,25 @@ __global__ void __launch_bounds__(256) gemm_merge_kernel(const GemmArgs g) {
     const int t = (int)blockIdx.x >> 4;
     const int wave = ((int)blockIdx.x >> 2) & 3, i = (int)blockIdx.x & 3;
     const int j = (int)threadIdx.x >> 6, lane = (int)threadIdx.x & 63;
+    // quad (tile row 2 i + (r >> 1), tile column 2 j + (r & 1)) for r < 4
     const f32x4* src = reinterpret_cast<const f32x4*>(g.part) +
-                       ((((int64_t)t * g.splits) * 4 + wave) * 64 + (16 * i + 4 * j)) * 64 + lane;
+                       ((((int64_t)t * g.splits) * 4 + wave) * 64 + (16 * i + 2 * j)) * 64 + lane;
     f32x4 v[kMaxKSplits][4];
 #pragma unroll
     for (int z = 0; z < kMaxKSplits; z++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             v[z][r] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (z < g.splits) v[z][r] = src[(int64_t)z * (4 * 64 * 64) + r * 64];
+            if (z < g.splits) v[z][r] = src[(int64_t)z * (4 * 64 * 64) + ((r >> 1) * 8 + (r & 1)) * 64];
         }
-    const int l32 = lane & 31, h = lane >> 5;
+    const int c16 = lane & 15, q4 = lane >> 4;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         f32x4 sum = v[0][r];
 #pragma unroll
         for (int z = 1; z < kMaxKSplits; z++)
             if (z < g.splits) sum += v[z][r];
-        unsigned char* dst = stage + l32 * PITCH + (32 * j + 8 * r + 4 * h) * ES;
+        unsigned char* dst = stage + (16 * (r >> 1) + c16) * PITCH + (32 * j + 16 * (r & 1) + 4 * q4) * ES;
         if constexpr (ES == 4) {
             *reinterpret_cast<f32x4*>(dst) = sum;
         } else {
