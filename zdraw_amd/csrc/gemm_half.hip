@@ -87,14 +87,16 @@ __device__ __forceinline__ f32x16 mfma(const u32x4& a, const u32x4& b, const f32
 // picks the three-address form for these 64 four-register accumulators and then moves them
 // around the accumulation file inside the loop (several copies per MFMA). The compiler inserts
 // no hazard waits around assembly: the caller keeps dependent MFMAs apart (here 64 MFMAs) and
-// calls mfma16_drain() before anything else reads the results.
+// calls mfma16_drain() in the same basic block as the last MFMA, before control can reach code
+// the compiler may have placed on its own (copies or spills of the accumulators at a join): a
+// result read within the MFMA's four passes is the old value.
 template <bool F16>
 __device__ __forceinline__ void mfma16(const u32x4& a, const u32x4& b, f32x4& c) {
     if constexpr (F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 __device__ __forceinline__ void mfma16_drain() {
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
 }
 
 // A wave's (32 TM) x (32 TN) block of C. The MFMAs take the W fragment as their first
@@ -237,8 +239,8 @@ __device__ __forceinline__ void store_tile16(const GemmArgs& g, void* c, const f
 // multiply. Staged rows are 256 bytes without padding; the 16-byte chunk c of row r sits at
 // c ^ (r & 15), which spreads both the 8-byte writes (16 rows x 2 halves per half wave) and the
 // row-wise reads over all banks. A wave's LDS operations complete in order, so the reads of one
-// pass see its writes and the next pass's writes follow its reads.
-// Needs 16-byte aligned rows of C.
+// pass see its writes and the next pass's writes follow its reads. Rows of C that do not start
+// on 16 bytes, and the columns past n, are stored element by element.
 constexpr int kEpiWaveBytes = 32 * 256;
 template <bool F16, typename TC>
 __device__ __forceinline__ void store_tile_lds16(const GemmArgs& g, void* c, const f32x4 (&acc)[8][8], unsigned lds_wave, int row0, int col0, int lane) {
@@ -252,7 +254,8 @@ __device__ __forceinline__ void store_tile_lds16(const GemmArgs& g, void* c, con
     // read: row 4 p + lane / 16 (p < 8), chunk lane % 16
     const int rr = lane >> 4, ch = lane & 15;
     const int col = col0 + 8 * ch;
-    const bool whole = col + 8 <= g.n;
+    // (uniform over the launch: rows of C start on 16 bytes; otherwise element by element)
+    const bool whole = col + 8 <= g.n && (g.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(c) % 16 == 0);
     unsigned short* const cbase = reinterpret_cast<unsigned short*>(c) + (int64_t)(row0 + rr) * g.ldc + col;
 #pragma unroll
     for (int ip = 0; ip < 4; ip++) {
@@ -266,6 +269,7 @@ __device__ __forceinline__ void store_tile_lds16(const GemmArgs& g, void* c, con
                 else pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
                 *(lds_u32x2_t)(wbase + (unsigned)(ii * 16 * 256) + (((unsigned)(2 * j) ^ wsw) * 16u)) = pk;
             }
+        __builtin_amdgcn_sched_barrier(0); // (keeps the scheduler from reading every accumulator out at once)
         u32x4 v[8];
 #pragma unroll
         for (int p2 = 0; p2 < 8; p2++) {
@@ -285,6 +289,7 @@ __device__ __forceinline__ void store_tile_lds16(const GemmArgs& g, void* c, con
                     if (col + e < g.n) dst[e] = (unsigned short)(v[p2][e >> 1] >> (16 * (e & 1)));
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -704,13 +709,14 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         mfma_step(std::false_type{}, I1{}, I0{}, f1, f0, s);
         mfma_step(std::true_type{}, I1{}, I1{}, f0, f1, s + 1);
         mfma_step(std::false_type{}, I0{}, I0{}, f1, f0, s + 1);
+        mfma16_drain(); // (24 cycles per two slabs: whatever follows the loop body may read the accumulators)
     }
     if (s < nslab) {
         mfma_step(std::true_type{}, I0{}, I1{}, f0, f1, s);
         mfma_step(std::false_type{}, I1{}, I0{}, f1, f0, s);
+        mfma16_drain();
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
-    mfma16_drain();
     if (g.splits > 1) {
         // partial tile in the accumulation layout: [tile][part][wave][i][j][lane] x 16 bytes,
         // every store instruction 1 KB in a row; the merge kernel reads it the same way
@@ -722,14 +728,10 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
             for (int j = 0; j < 8; j++) dst[(i * 8 + j) * 64] = acc[i][j];
         return;
     }
-    if constexpr (sizeof(TC) == 2) {
-        // uniform over the launch: rows of C start on 16 bytes
-        if ((g.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(cp) % 16 == 0)) {
-            store_tile_lds16<F16, TC>(g, cp, acc, lds0 + 2u * DMA_STAGE_BYTES + (unsigned)wave * kEpiWaveBytes, m0 + wm * 128, n0 + wn * 128, lane);
-            return;
-        }
-    }
-    store_tile16<F16, TC>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, lane);
+    if constexpr (sizeof(TC) == 2)
+        store_tile_lds16<F16, TC>(g, cp, acc, lds0 + 2u * DMA_STAGE_BYTES + (unsigned)wave * kEpiWaveBytes, m0 + wm * 128, n0 + wn * 128, lane);
+    else
+        store_tile16<F16, TC>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, lane);
 }
 
 // Adds the parts of the k-split tiles in part order and writes C. A workgroup takes the 32 x
