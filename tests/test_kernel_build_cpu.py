@@ -1,0 +1,21 @@
+"""Build-level checks of the hand-written kernels that need no GPU.
+
+The four-wave GEMM issues its v_mfma_f32_16x16x32 instructions as assembly
+statements with the accumulator tied to the result (zdraw_amd/csrc/gemm_half.hip,
+mfma16). The compiler adds no wait states around assembly, so anything it places
+on its own between such an MFMA and the `s_nop 15` that ends the run (a copy or a
+spill of an accumulator) would read the register before the MFMA has written it.
+The check compiles the file to gfx950 assembly and fails on any such instruction.
+"""
+import os
+import shutil
+
+import pytest
+
+from zdraw_amd import build
+
+
+@pytest.mark.skipif(not (os.path.exists("/opt/rocm/bin/hipcc") or shutil.which("hipcc")), reason="needs hipcc")
+def test_nothing_reads_an_accumulator_inside_a_run_of_tied_mfmas():
+    bad = build.tied_mfma_hazards()
+    assert not bad, "\n".join(bad[:20])

@@ -55,6 +55,42 @@ def build_hip(verbose: bool = False, out: str | None = None, extra_flags=()) -> 
     return target
 
 
+def tied_mfma_hazards(src: str = os.path.join(CSRC, "gemm_half.hip"), extra_flags=()) -> list[str]:
+    """Compiles `src` to gfx950 assembly and lists every place where something other than
+    an MFMA touches an accumulation register while a hand-written v_mfma_f32_16x16x32 may
+    still be writing it. Those MFMAs are assembly statements, so the compiler adds none of
+    the wait states it adds after the builtin; the source instead ends every run of them
+    with `s_nop 15` before control leaves the block. A copy or spill of an accumulator that
+    the register allocator places inside such a run would read a stale value: this check
+    (run by the CPU tests) fails the build that contains one."""
+    import re
+    import tempfile
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, "out.s")
+        _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-S", "--cuda-device-only", "-o", asm, src])
+        with open(asm) as f:
+            lines = f.read().split("\n")
+    bad = []
+    agpr = re.compile(r"\ba(\[\d+:\d+\]|\d+)\b")
+    kernel, hot = "", False
+    for no, line in enumerate(lines, 1):
+        text = line.split(";")[0].strip()
+        if not text:
+            continue
+        if text.endswith(":") and not text.startswith("."):
+            kernel, hot = text[:-1], False
+            continue
+        op = text.split()[0]
+        if op.startswith("v_mfma_f32_16x16x32"):
+            hot = True
+        elif op == "s_nop" and text.split()[1] == "15":
+            hot = False
+        elif hot and agpr.search(text):
+            bad.append(f"{kernel}: line {no}: {text}")
+    return bad
+
+
 def build_host(verbose: bool = False) -> str:
     os.makedirs(LIBDIR, exist_ok=True)
     srcs = [os.path.join(HOST, f) for f in sorted(os.listdir(HOST)) if f.endswith(".cc")]
