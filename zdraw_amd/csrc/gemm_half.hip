@@ -6,8 +6,9 @@
 // (metal/mgemm_shader.zig, metal_api.m) that produce Q, K, V from the block
 // input and drain the attention output (klein/zflux2_resident.zig:1473-1513,
 // 1986-1998). Both operands are K-major (activation rows and weight rows are
-// contiguous in k), which is exactly the register layout of
-// v_mfma_f32_32x32x16: a lane supplies 8 consecutive k of one row.
+// contiguous in k), which is exactly the register layout of the 16-bit MFMAs
+// (v_mfma_f32_16x16x32 in the direct-to-LDS builds, v_mfma_f32_32x32x16 in the
+// register-staged one): a lane supplies 8 consecutive k of one row.
 //
 // Three builds share the tile walk, the operand layout and the epilogue:
 //   * f32 activations, or k not a multiple of 64: workgroup tile 256 x 256, K slabs of
@@ -22,7 +23,8 @@
 //   * the same with too few 256-tiles: 128 x 128 tiles, 4 waves, two workgroups per CU;
 //   * two or three products of one A with equal shapes (q/k/v, gate/up) run as one launch
 //     whose tiles cover all of them;
-//   * fixed summation order, no split-K, no atomics: bit-identical run to run.
+//   * fixed summation order and no atomics (a thinly filled last round is cut along k and
+//     merged in part order): bit-identical run to run.
 #include "attn_device.hpp"
 #include "gemm_kernel.h"
 
@@ -138,82 +140,21 @@ __device__ __forceinline__ void store_tile(const GemmArgs& g, void* c, const f32
     }
 }
 
-// The same block of C for a 16-bit C, by way of LDS: stored straight from the accumulation
-// layout a lane's 8 bytes make every store instruction 32 separate 16-byte pieces; turned
-// through a wave-private region of the (by then idle) slab stages, (32 TM) rows of
-// epi_pitch(TN) bytes, every instruction stores whole rows of the block (four 256-byte rows
-// for TN = 4, eight 128-byte rows for TN = 2).
-// Needs: every direct load of the workgroup has landed and a barrier has passed since the last
-// fragment read; 16-byte aligned rows of C.
-constexpr int epi_pitch(int tn) { return 64 * tn + 16; } // bytes per staged row: keeps 16-byte alignment, spreads the banks
-template <bool F16, typename TC, int TM, int TN>
-__device__ __forceinline__ void store_tile_lds(const GemmArgs& g, void* c, const f32x16 (&acc)[TM][TN], unsigned lds_wave, int row0, int col0, int lane) {
-    static_assert(sizeof(TC) == 2, "16-bit C only");
-    constexpr int PITCH = epi_pitch(TN);
-    constexpr int CH = 4 * TN;   // 16-byte chunks per staged row
-    constexpr int RPI = 64 / CH; // rows per read-back instruction
-    constexpr int NQ = 32 * TM / RPI;
-    typedef __attribute__((address_space(3))) u32x2* lds_u32x2_t;
-    typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
-    const int l32 = lane & 31, h = lane >> 5;
-    const unsigned wbase = lds_wave + (unsigned)(l32 * PITCH + h * 8);
-#pragma unroll
-    for (int i = 0; i < TM; i++) {
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const f32x4 v = f32x4{acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2], acc[i][j][4 * r + 3]};
-                u32x2 pk;
-                if constexpr (F16) pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4));
-                else pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
-                *(lds_u32x2_t)(wbase + (unsigned)(i * 32 * PITCH + j * 64 + r * 16)) = pk;
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    // lane -> row RPI q + lane / CH, columns 8 (lane % CH) .. + 8
-    const int rr = lane / CH, ch = lane % CH;
-    const int col = col0 + 8 * ch;
-    const unsigned rbase = lds_wave + (unsigned)(rr * PITCH + ch * 16);
-    unsigned short* const cbase = reinterpret_cast<unsigned short*>(c) + (int64_t)(row0 + rr) * g.ldc + col;
-    const bool whole = col + 8 <= g.n;
-#pragma unroll
-    for (int q0 = 0; q0 < NQ; q0 += 8) {
-        u32x4 v[8];
-#pragma unroll
-        for (int q = 0; q < 8; q++) v[q] = *(lds_u32x4_t)(rbase + (unsigned)((q0 + q) * RPI * PITCH));
-#pragma unroll
-        for (int q = 0; q < 8; q++) {
-            const int row = row0 + RPI * (q0 + q) + rr;
-            if (row >= g.m) continue;
-            unsigned short* const dst = cbase + (int64_t)(RPI * (q0 + q)) * g.ldc;
-            if (whole) {
-                *reinterpret_cast<u32x4*>(dst) = v[q];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; e++)
-                    if (col + e < g.n) dst[e] = (unsigned short)(v[q][e >> 1] >> (16 * (e & 1)));
-            }
-        }
-    }
-}
-
-// The four-wave build's block of C: 8 x 8 tiles of 16 x 16. The MFMAs take the W fragment as
+// A wave's (16 TI) x (16 TJ) block of C from 16 x 16 x 32 MFMAs. They take the W fragment as
 // their first operand, so a lane (c = lane % 16, q = lane / 16) holds row row0 + 16 i + c of C
 // and, in tile (i, j), columns col0 + 16 j + 4 q .. + 3: a store instruction covers 16 rows x 64
 // contiguous bytes of f32.
-template <bool F16, typename TC>
-__device__ __forceinline__ void store_tile16(const GemmArgs& g, void* c, const f32x4 (&acc)[8][8], int row0, int col0, int lane) {
+template <bool F16, typename TC, int TI, int TJ>
+__device__ __forceinline__ void store_tile16(const GemmArgs& g, void* c, const f32x4 (&acc)[TI][TJ], int row0, int col0, int lane) {
     const int c16 = lane & 15, q = lane >> 4;
     const bool vec = (g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(c) % (4 * sizeof(TC))) == 0);
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < TI; i++) {
         const int row = row0 + 16 * i + c16;
         if (row >= g.m) continue;
         TC* const crow = reinterpret_cast<TC*>(c) + (int64_t)row * g.ldc;
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
+        for (int j = 0; j < TJ; j++) {
             const int col = col0 + 16 * j + 4 * q;
             const f32x4 v = acc[i][j];
             if (vec && col + 4 <= g.n) {
@@ -233,54 +174,61 @@ __device__ __forceinline__ void store_tile16(const GemmArgs& g, void* c, const f
     }
 }
 
-// The same block for a 16-bit C, as whole 256-byte rows: the wave turns 32 rows at a time (two
-// rows of tiles) through 8 KB of LDS that are its own and lie behind the slab stages, so no
-// barrier is needed and a wave that finishes its last slab early stores while the others still
-// multiply. Staged rows are 256 bytes without padding; the 16-byte chunk c of row r sits at
-// c ^ (r & 15), which spreads both the 8-byte writes (16 rows x 2 halves per half wave) and the
-// row-wise reads over all banks. A wave's LDS operations complete in order, so the reads of one
-// pass see its writes and the next pass's writes follow its reads. Rows of C that do not start
-// on 16 bytes, and the columns past n, are stored element by element.
+// The same block for a 16-bit C, as whole rows of the block (32 TJ bytes: 256 for TJ = 8, 128
+// for TJ = 4): the wave turns 32 rows at a time (two rows of tiles) through LDS of its own
+// (32 x 32 TJ bytes at lds_wave), so it needs no barrier of its own; the caller sees to it that
+// nobody else uses that LDS any more. Staged rows are unpadded; the 16-byte chunk c of row r
+// sits at c ^ (r & 15) in 256-byte rows and at c ^ ((r >> 1) & 7) in 128-byte rows, which
+// spreads both the 8-byte writes (16 rows x 2 halves per half wave) and the row-wise reads over
+// all banks. A wave's LDS operations complete in order, so the reads of one pass see its
+// writes and the next pass's writes follow its reads. Rows of C that do not start on 16 bytes,
+// and the columns past n, are stored element by element.
 constexpr int kEpiWaveBytes = 32 * 256;
-template <bool F16, typename TC>
-__device__ __forceinline__ void store_tile_lds16(const GemmArgs& g, void* c, const f32x4 (&acc)[8][8], unsigned lds_wave, int row0, int col0, int lane) {
+template <bool F16, typename TC, int TI, int TJ>
+__device__ __forceinline__ void store_tile_lds16(const GemmArgs& g, void* c, const f32x4 (&acc)[TI][TJ], unsigned lds_wave, int row0, int col0, int lane) {
     static_assert(sizeof(TC) == 2, "16-bit C only");
+    static_assert((TJ == 8 || TJ == 4) && TI % 2 == 0, "blocks of 128 or 64 columns, rows in pairs of tiles");
+    constexpr int ROWB = 32 * TJ;   // bytes per staged row
+    constexpr int NCH = 2 * TJ;     // 16-byte chunks per row
+    constexpr int RPI = 64 / NCH;   // rows per read-back instruction
     typedef __attribute__((address_space(3))) u32x2* lds_u32x2_t;
     typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
+    auto swz = [](int r) { return TJ == 8 ? (r & 15) : ((r >> 1) & 7); };
     const int c16 = lane & 15, q = lane >> 4;
     // write: row 16 (i & 1) + c16, bytes 32 j + 8 q .. + 8 = chunk 2 j + q / 2, half q & 1
-    const unsigned wbase = lds_wave + (unsigned)(c16 * 256 + (q & 1) * 8);
-    const unsigned wsw = (unsigned)(c16 ^ (q >> 1)); // (2 j + q / 2) ^ c16 = (2 j) ^ (c16 ^ (q / 2))
-    // read: row 4 p + lane / 16 (p < 8), chunk lane % 16
-    const int rr = lane >> 4, ch = lane & 15;
+    const unsigned wbase = lds_wave + (unsigned)(c16 * ROWB + (q & 1) * 8);
+    const unsigned wsw = (unsigned)(swz(c16) ^ (q >> 1)); // (2 j + q / 2) ^ s = (2 j) ^ (s ^ (q / 2))
+    // read: row RPI p + lane / NCH (p < 32 / RPI), chunk lane % NCH
+    const int rr = lane / NCH, ch = lane % NCH;
     const int col = col0 + 8 * ch;
     // (uniform over the launch: rows of C start on 16 bytes; otherwise element by element)
     const bool whole = col + 8 <= g.n && (g.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(c) % 16 == 0);
     unsigned short* const cbase = reinterpret_cast<unsigned short*>(c) + (int64_t)(row0 + rr) * g.ldc + col;
 #pragma unroll
-    for (int ip = 0; ip < 4; ip++) {
+    for (int ip = 0; ip < TI / 2; ip++) {
 #pragma unroll
         for (int ii = 0; ii < 2; ii++)
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
+            for (int j = 0; j < TJ; j++) {
                 const f32x4 v = acc[2 * ip + ii][j];
                 u32x2 pk;
                 if constexpr (F16) pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4));
                 else pk = __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
-                *(lds_u32x2_t)(wbase + (unsigned)(ii * 16 * 256) + (((unsigned)(2 * j) ^ wsw) * 16u)) = pk;
+                // (rows 16 .. 31 swizzle as rows 0 .. 15 do: both forms of swz ignore bit 4)
+                *(lds_u32x2_t)(wbase + (unsigned)(ii * 16 * ROWB) + (((unsigned)(2 * j) ^ wsw) * 16u)) = pk;
             }
         __builtin_amdgcn_sched_barrier(0); // (keeps the scheduler from reading every accumulator out at once)
-        u32x4 v[8];
+        u32x4 v[32 / RPI];
 #pragma unroll
-        for (int p2 = 0; p2 < 8; p2++) {
-            const int r = 4 * p2 + rr;
-            v[p2] = *(lds_u32x4_t)(lds_wave + (unsigned)(r * 256) + (unsigned)((ch ^ (r & 15)) * 16));
+        for (int p2 = 0; p2 < 32 / RPI; p2++) {
+            const int r = RPI * p2 + rr;
+            v[p2] = *(lds_u32x4_t)(lds_wave + (unsigned)(r * ROWB) + (unsigned)((ch ^ swz(r)) * 16));
         }
 #pragma unroll
-        for (int p2 = 0; p2 < 8; p2++) {
-            const int row = row0 + 32 * ip + 4 * p2 + rr;
+        for (int p2 = 0; p2 < 32 / RPI; p2++) {
+            const int row = row0 + 32 * ip + RPI * p2 + rr;
             if (row >= g.m) continue;
-            unsigned short* const dst = cbase + (int64_t)(32 * ip + 4 * p2) * g.ldc;
+            unsigned short* const dst = cbase + (int64_t)(32 * ip + RPI * p2) * g.ldc;
             if (whole) {
                 *reinterpret_cast<u32x4*>(dst) = v[p2];
             } else {
@@ -459,7 +407,7 @@ template <bool F16, typename TC, int WM, int WN, int TB>
 __global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArgs g) {
     constexpr int STAGE_BYTES = 2 * TB * BK * 2; // A rows then W rows
     constexpr int NW = WM * WN;
-    constexpr int TM = TB / WM / 32, TN = TB / WN / 32; // 32 x 32 MFMA tiles per wave
+    constexpr int TM = TB / WM / 16, TN = TB / WN / 16; // 16 x 16 MFMA tiles per wave
     constexpr int RW = TB / NW;                           // slab rows a wave fetches, of A and of W
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -467,8 +415,8 @@ __global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArg
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int l32 = lane & 31;
-    const int h = lane >> 5;
+    const int c16 = lane & 15;
+    const int q4 = lane >> 4;
     const int wm = wave / WN, wn = wave % WN;
     const int logical = logical_tile();
     const int tiles_row = g.tiles_n * g.groups;
@@ -507,32 +455,37 @@ __global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArg
         }
     };
 
-    f32x16 acc[TM][TN];
+    f32x4 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+        for (int j = 0; j < TN; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // fragment addresses: row (.. + l32), logical chunk 2 kk + h at position (2 kk + h) ^ ((l32 >> 1) & 7)
-    const int sw = (l32 >> 1) & 7;
-    const int a_row = (wm * (32 * TM) + l32) * (BK * 2);
-    const int w_row = TB * BK * 2 + (wn * (32 * TN) + l32) * (BK * 2);
+    // fragment addresses: row (.. + c16), logical chunk 4 ks + q4 at position (4 ks + q4) ^ ((c16 >> 1) & 7)
+    const int sw = (c16 >> 1) & 7;
+    const int a_row = (wm * (16 * TM) + c16) * (BK * 2);
+    const int w_row = TB * BK * 2 + (wn * (16 * TN) + c16) * (BK * 2);
     struct Frag { u32x4 a[TM], w[TN]; };
-    auto read_frag = [&](Frag& f, int s, int kk) __attribute__((always_inline)) {
+    auto read_frag = [&](Frag& f, int s, int ks) __attribute__((always_inline)) {
         const unsigned char* st = smem + (s & 1) * STAGE_BYTES;
-        const int pos = ((2 * kk + h) ^ sw) * 16;
+        const int pos = ((4 * ks + q4) ^ sw) * 16;
 #pragma unroll
-        for (int i = 0; i < TM; i++) f.a[i] = *reinterpret_cast<const u32x4*>(st + a_row + i * 32 * (BK * 2) + pos);
+        for (int i = 0; i < TM; i++) f.a[i] = *reinterpret_cast<const u32x4*>(st + a_row + i * 16 * (BK * 2) + pos);
 #pragma unroll
-        for (int j = 0; j < TN; j++) f.w[j] = *reinterpret_cast<const u32x4*>(st + w_row + j * 32 * (BK * 2) + pos);
+        for (int j = 0; j < TN; j++) f.w[j] = *reinterpret_cast<const u32x4*>(st + w_row + j * 16 * (BK * 2) + pos);
     };
+    // (The builtin form: with this few accumulators the compiler keeps them in place, and it
+    // adds the wait states itself.)
     auto mfma_frag = [&](const Frag& f) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) acc[i][j] = mfma<F16>(f.w[j], f.a[i], acc[i][j]);
+            for (int j = 0; j < TN; j++) {
+                if constexpr (F16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, f.w[j]), __builtin_bit_cast(f16x8, f.a[i]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, f.w[j]), __builtin_bit_cast(bf16x8, f.a[i]), acc[i][j], 0, 0, 0);
+            }
     };
 
     fetch_slab(0);
@@ -544,24 +497,22 @@ __global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArg
         // then makes the fragment reads that follow each load wait for it.)
         if (s + 1 < nslab) fetch_slab(s + 1);
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; kk++) {
+        for (int ks = 0; ks < BK / 32; ks++) {
             Frag f;
-            read_frag(f, s, kk);
+            read_frag(f, s, ks);
             mfma_frag(f);
         }
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): slab s+1 has landed
         __syncthreads();
     }
     if constexpr (sizeof(TC) == 2 && TB == 128) {
-        // the loop's last barrier has left the stages idle; the staged tile fits into them
-        static_assert((size_t)WM * WN * 32 * TM * epi_pitch(TN) <= 2 * (size_t)(2 * TB * BK * 2), "staging exceeds the slab stages");
-        if ((g.ldc % 8 == 0) && (reinterpret_cast<uintptr_t>(cp) % 16 == 0)) {
-            store_tile_lds<F16, TC, TM, TN>(g, cp, acc, lds_address(smem) + (unsigned)wave * (32 * TM * epi_pitch(TN)),
-                                            m0 + wm * (32 * TM), n0 + wn * (32 * TN), lane);
-            return;
-        }
+        // the loop's last barrier has left the stages idle; each wave stages 32 rows of its block in them
+        static_assert((size_t)WM * WN * 32 * (32 * TN) <= 2 * (size_t)(2 * TB * BK * 2), "staging exceeds the slab stages");
+        store_tile_lds16<F16, TC, TM, TN>(g, cp, acc, lds_address(smem) + (unsigned)wave * (32 * 32 * TN),
+                                          m0 + wm * (16 * TM), n0 + wn * (16 * TN), lane);
+    } else {
+        store_tile16<F16, TC, TM, TN>(g, cp, acc, m0 + wm * (16 * TM), n0 + wn * (16 * TN), lane);
     }
-    store_tile<F16, TC, TM, TN>(g, cp, acc, m0 + wm * (32 * TM), n0 + wn * (32 * TN), l32, h);
 }
 
 // ---------------------------------------------------------------------------
@@ -729,9 +680,9 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         return;
     }
     if constexpr (sizeof(TC) == 2)
-        store_tile_lds16<F16, TC>(g, cp, acc, lds0 + 2u * DMA_STAGE_BYTES + (unsigned)wave * kEpiWaveBytes, m0 + wm * 128, n0 + wn * 128, lane);
+        store_tile_lds16<F16, TC, 8, 8>(g, cp, acc, lds0 + 2u * DMA_STAGE_BYTES + (unsigned)wave * kEpiWaveBytes, m0 + wm * 128, n0 + wn * 128, lane);
     else
-        store_tile16<F16, TC>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, lane);
+        store_tile16<F16, TC, 8, 8>(g, cp, acc, m0 + wm * 128, n0 + wn * 128, lane);
 }
 
 // Adds the parts of the k-split tiles in part order and writes C. A workgroup takes the 32 x
