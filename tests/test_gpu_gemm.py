@@ -354,6 +354,36 @@ def test_many_tile_problem_runs_the_256_tile_builds(ctx, build, c_dtype, a32):
     assert np.abs(got[-1] - want[-1]).max() < tol and np.abs(got[:, -1] - want[:, -1]).max() < tol
 
 
+@pytest.mark.parametrize("build", [1, 0])
+def test_256_tile_builds_16_bit_output_with_unaligned_rows(ctx, build):
+    # the same 169 tiles with a pitch of 3291 elements: no row of C starts on 16 bytes, so every
+    # 16-bit store is made element by element (four waves: after the turn through LDS; eight
+    # waves: from the registers); the pad column of the pitch and the guard behind the last row
+    # stay untouched
+    L = hip.lib()
+    rng = np.random.default_rng(29)
+    m, k, n, ldc = 3300, 128, 3290, 3291
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
+    a_bits, ar = to16(a, hip.W_BF16)
+    w_bits, wr = to16(w, hip.W_BF16)
+    guard = 64
+    init = np.full(m * ldc + guard, 0x7e7e, np.uint16)
+    L.zdraw_hip_set_gemm_build(build)
+    try:
+        raw = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, hip.BF16, ldc=ldc, c_init=init.view(np.uint8))
+    finally:
+        L.zdraw_hip_set_gemm_build(1)
+    flat = raw.view(np.uint16)
+    assert (flat[m * ldc:] == 0x7e7e).all()
+    full = flat[:m * ldc].reshape(m, ldc)
+    assert (full[:, n:] == 0x7e7e).all()
+    got = from16(full[:, :n], hip.W_BF16)
+    want = zo.linear_batch(ar, wr)
+    s = np.sqrt(k) * np.sqrt(np.mean(ar.astype(np.float64) ** 2)) * np.sqrt(np.mean(wr.astype(np.float64) ** 2))
+    assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max() + 2e-5 * s  # one bf16 rounding of the fp32 result
+
+
 @pytest.mark.parametrize("wdt", [hip.W_BF16, hip.W_F16])
 @pytest.mark.parametrize("ldc", [256, 251])
 def test_small_tile_build_16_bit_output_edges_and_pitch(ctx, wdt, ldc):
