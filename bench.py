@@ -253,7 +253,7 @@ def gemm_main(args):
     for b in (ab, wb, cb):
         b.release()
     ctx.deinit()
-    print(json.dumps(line), flush=True)
+    return line
 
 
 def chain_main(args):
@@ -338,7 +338,7 @@ def chain_main(args):
     for b in (nb, wb, qb, kb, vb, mixb, ob, ones, posb, ropeb):
         b.release()
     ctx.deinit()
-    print(json.dumps(line), flush=True)
+    return line
 
 
 def wide_main(args):
@@ -383,6 +383,8 @@ def wide_main(args):
     burst(args.steps)
     wall = time.perf_counter() - t0
     # the attention kernel alone: its own HIP events on the launch stream
+    L.zdraw_hip_queue_sync(ctx.queue)
+    L.zdraw_hip_metrics_reset()  # (the totals are the process's: an earlier leg may have traced too)
     L.zdraw_hip_trace_attention(1)
     burst(args.steps)
     launches = C.c_uint64(0)
@@ -423,7 +425,25 @@ def wide_main(args):
     for b in (qb, kb, vb, ob):
         b.release()
     ctx.deinit()
-    print(json.dumps(line), flush=True)
+    return line
+
+
+PATH_MAINS = {"gemm": gemm_main, "chain": chain_main, "wide": wide_main}
+
+
+def other_paths(args):
+    """Short legs of the other kernels on this path's either side (`--path gemm|chain|wide` at their
+    default shapes), outside the driver-timed region, for the record in the same line."""
+    import copy
+
+    out = {}
+    for name, steps in (("gemm", 200), ("chain", 60), ("wide", 60)):
+        a = copy.copy(args)
+        a.path, a.steps, a.warmup, a.spinup_ms, a.no_cpu = name, steps, 10, 400.0, True
+        line = PATH_MAINS[name](a)
+        out[name] = {"workload": line["config"]["workload"], "value": line["value"], "ms_per_step": line["ms_per_step"],
+                     "kernel_frac": line["roofline"]["frac"], "kernel": line["roofline"]["kernel"]}
+    return out
 
 
 def main():
@@ -450,7 +470,7 @@ def main():
     ap.add_argument("--dynamic-max", action="store_true", help="withhold the score bound (running-maximum softmax)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-side-legs", action="store_true",
-                    help="skip the short untimed-by-value legs (other softmax form, other benchmark shapes)")
+                    help="skip the short untimed-by-value legs (other softmax form, other benchmark shapes, the GEMM, chain and wide-head paths)")
     ap.add_argument("--cu-count", type=int, default=0,
                     help="confine the library's stream to this many compute units (0 = all): shows whether "
                          "the kernel's time follows the CU count or the board's power limit")
@@ -462,12 +482,9 @@ def main():
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)")
     if args.cu_count > 0:
         os.environ["ZDRAW_HIP_CU_COUNT"] = str(args.cu_count)  # read when the library creates its stream
-    if args.path == "gemm":
-        return gemm_main(args)
-    if args.path == "chain":
-        return chain_main(args)
-    if args.path == "wide":
-        return wide_main(args)
+    if args.path in PATH_MAINS:
+        print(json.dumps(PATH_MAINS[args.path](args)), flush=True)
+        return
     if args.workload == "attn_scale":
         return attn_scale_main(args)
 
@@ -585,6 +602,8 @@ def main():
         },
     }
     ctx.deinit()
+    if not args.no_side_legs:
+        line["config"]["other_paths"] = other_paths(args)
     if args.copy_calibration_mib:
         import torch
 
