@@ -354,6 +354,23 @@ def test_many_tile_problem_runs_the_256_tile_builds(ctx, build, c_dtype, a32):
     assert np.abs(got[-1] - want[-1]).max() < tol and np.abs(got[:, -1] - want[:, -1]).max() < tol
 
 
+@pytest.mark.parametrize("k", [64, 192, 320])
+def test_four_wave_build_with_one_three_and_five_slabs(ctx, k):
+    # the four-wave loop takes two slabs per trip and requests slabs two ahead: one slab (no
+    # trip, the odd tail only), three and five (trips plus the tail), 169 tiles each
+    rng = np.random.default_rng(31 + k)
+    m, n = 3300, 3290
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
+    a_bits, ar = to16(a, hip.W_BF16)
+    w_bits, wr = to16(w, hip.W_BF16)
+    raw = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, hip.F32)
+    got = raw.view(np.float32).reshape(m, n)
+    check(got, zo.linear_batch(ar, wr), zo.linear_batch(a, w), k, a, w, f"k = {k}")
+    again = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, hip.F32)
+    assert np.array_equal(raw, again)
+
+
 @pytest.mark.parametrize("build", [1, 0])
 def test_256_tile_builds_16_bit_output_with_unaligned_rows(ctx, build):
     # the same 169 tiles with a pitch of 3291 elements: no row of C starts on 16 bytes, so every
