@@ -19,3 +19,11 @@ from zdraw_amd import build
 def test_nothing_reads_an_accumulator_inside_a_run_of_tied_mfmas():
     bad = build.tied_mfma_hazards()
     assert not bad, "\n".join(bad[:20])
+
+
+@pytest.mark.skipif(not (os.path.exists("/opt/rocm/bin/hipcc") or shutil.which("hipcc")), reason="needs hipcc")
+def test_only_the_source_writes_m0_in_the_four_wave_gemm():
+    # its slab loads come in runs of four that share one M0 (attn_device.hpp, lds_dma_base): the
+    # compiler does not know M0 is live between them, so it must not have put a write of its own there
+    bad = build.m0_writes()
+    assert not bad, "\n".join(bad[:20])

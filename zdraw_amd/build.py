@@ -55,6 +55,40 @@ def build_hip(verbose: bool = False, out: str | None = None, extra_flags=()) -> 
     return target
 
 
+def _device_asm(src: str, extra_flags=()) -> list[str]:
+    import tempfile
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, "out.s")
+        _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-S", "--cuda-device-only", "-o", asm, src])
+        with open(asm) as f:
+            return f.read().split("\n")
+
+
+def m0_writes(src: str = os.path.join(CSRC, "gemm_half.hip"), kernel_substr: str = "gemm_ring_kernel", extra_flags=()) -> list[str]:
+    """Compiles `src` to gfx950 assembly and lists, for the kernels whose symbol contains
+    `kernel_substr`, every instruction that writes M0 other than the source's own
+    `s_mov_b32 m0, <sgpr>` + `s_nop 0` pair (attn_device.hpp, lds_dma_base). The four-wave GEMM
+    keeps M0 live across several loads without the compiler knowing; a write of the compiler's
+    own in between would send those loads elsewhere in LDS."""
+    import re
+    lines = [l.split(";")[0].strip() for l in _device_asm(src, extra_flags)]
+    lines = [l for l in lines if l]
+    bad = []
+    kernel = ""
+    writes = re.compile(r"^s_\w+\s+m0\s*,")
+    for i, text in enumerate(lines):
+        if text.endswith(":") and not text.startswith("."):
+            kernel = text[:-1]
+            continue
+        if kernel_substr not in kernel or not writes.match(text):
+            continue
+        own = re.match(r"^s_mov_b32\s+m0\s*,\s*s\d+$", text) and i + 1 < len(lines) and lines[i + 1] == "s_nop 0"
+        if not own:
+            bad.append(f"{kernel}: {text}")
+    return bad
+
+
 def tied_mfma_hazards(src: str = os.path.join(CSRC, "gemm_half.hip"), extra_flags=()) -> list[str]:
     """Compiles `src` to gfx950 assembly and lists every place where something other than
     an MFMA touches an accumulation register while a hand-written v_mfma_f32_16x16x32 may
@@ -64,13 +98,7 @@ def tied_mfma_hazards(src: str = os.path.join(CSRC, "gemm_half.hip"), extra_flag
     the register allocator places inside such a run would read a stale value: this check
     (run by the CPU tests) fails the build that contains one."""
     import re
-    import tempfile
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    with tempfile.TemporaryDirectory() as tmp:
-        asm = os.path.join(tmp, "out.s")
-        _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-S", "--cuda-device-only", "-o", asm, src])
-        with open(asm) as f:
-            lines = f.read().split("\n")
+    lines = _device_asm(src, extra_flags)
     bad = []
     agpr = re.compile(r"\ba(\[\d+:\d+\]|\d+)\b")
     kernel, hot = "", False

@@ -83,6 +83,22 @@ __device__ __forceinline__ void load_to_lds_16(u32x4 rsrc, unsigned lds_addr, un
                  : "memory", "m0");
 }
 
+// The same load in two parts, for runs of loads whose LDS targets differ by less than 4 KB:
+// lds_dma_base sets M0 once, load_to_lds_16_at<IMM> adds IMM (< 4096) to it. The instruction's
+// offset field moves the address in memory by IMM as well: the caller takes it off thread_off
+// (biasing the descriptor's base downwards keeps that offset from going negative). M0 has to
+// stay as it is between the parts; the compiler does not know that it is live, so a kernel that
+// uses the pair may contain nothing else that writes M0 (zdraw_amd.build.m0_writes lists what a
+// compiled file holds).
+__device__ __forceinline__ void lds_dma_base(unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_addr) : "memory", "m0");
+}
+template <int IMM>
+__device__ __forceinline__ void load_to_lds_16_at(u32x4 rsrc, unsigned thread_off, unsigned uniform_off) {
+    static_assert(IMM >= 0 && IMM < 4096, "12-bit instruction offset");
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds" : : "v"(thread_off), "s"(rsrc), "s"(uniform_off), "n"(IMM) : "memory");
+}
+
 __device__ __forceinline__ void unpack8(const Raw8<float>& r, float (&x)[8]) {
 #pragma unroll
     for (int i = 0; i < 4; i++) { x[i] = r.a[i]; x[4 + i] = r.b[i]; }

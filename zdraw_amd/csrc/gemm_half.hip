@@ -559,8 +559,13 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
 
     const unsigned a_span = ((unsigned)(g.m - 1) * (unsigned)g.lda + (unsigned)g.k) * 2u;
     const unsigned w_span = ((unsigned)(g.n - 1) * (unsigned)g.ldw + (unsigned)g.k) * 2u;
-    const u32x4 a_rsrc = make_rsrc_words(g.a, a_span);
-    const u32x4 w_rsrc = make_rsrc_words(wp, w_span);
+    // The 16 loads of a slab go as four runs of four whose LDS targets lie 1 KB apart: M0 is set
+    // once per run and the other three use the instruction's offset field, which also moves the
+    // address in memory; that is taken off the lane's offset, and the descriptors start 3 KB
+    // below the operands so that the offset stays positive.
+    constexpr unsigned kBias = 3 * 1024;
+    const u32x4 a_rsrc = make_rsrc_words(reinterpret_cast<const unsigned char*>(g.a) - kBias, a_span + kBias);
+    const u32x4 w_rsrc = make_rsrc_words(reinterpret_cast<const unsigned char*>(wp) - kBias, w_span + kBias);
     const unsigned lds0 = lds_address(smem);
     // wave w fills rows 64 w + 8 j + lane / 8 (j < 8) of the A slab and of the W slab
     unsigned a_off[8], w_off[8];
@@ -570,8 +575,8 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         const int c = (lane & 7) ^ ((r >> 1) & 7);
         const int ar = min(m0 + r, g.m - 1); // rows past the edge re-read the last row; never stored
         const int wr = min(n0 + r, g.n - 1);
-        a_off[j] = ((unsigned)ar * (unsigned)g.lda + (unsigned)(c * 8)) * 2u;
-        w_off[j] = ((unsigned)wr * (unsigned)g.ldw + (unsigned)(c * 8)) * 2u;
+        a_off[j] = ((unsigned)ar * (unsigned)g.lda + (unsigned)(c * 8)) * 2u + kBias - (unsigned)(j & 3) * 1024u;
+        w_off[j] = ((unsigned)wr * (unsigned)g.ldw + (unsigned)(c * 8)) * 2u + kBias - (unsigned)(j & 3) * 1024u;
     }
     int nslab = g.k / BK, slab0 = 0;
     if (g.splits > 1) {
@@ -581,13 +586,21 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
     }
     const unsigned fetch_lds = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)wave * (64 * BK * 2));
     // slabs past the end re-fetch the last slab into a stage nobody reads any more
-    // the i-th (i < 16) of the loads that bring this wave's part of slab s in
+    // the i-th (i < 16) of the loads that bring this wave's part of slab s in, in the order A rows
+    // 0..31 of the wave's 64, W rows 0..31, A rows 32..63, W rows 32..63 (eight rows a load); the
+    // loads of a run must be issued in order, the first sets M0 for the rest
     auto fetch_one = [&](int s, int i) __attribute__((always_inline)) {
         const unsigned uo = (unsigned)min(slab0 + max(s < nslab ? s : nslab - 1, 0), g.k / BK - 1) * (BK * 2u);
-        const unsigned base = fetch_lds + (unsigned)(s & 1) * DMA_STAGE_BYTES;
-        const int j = i >> 1;
-        if ((i & 1) == 0) load_to_lds_16(a_rsrc, base + (unsigned)j * (8 * BK * 2), a_off[j], uo);
-        else load_to_lds_16(w_rsrc, base + BM * BK * 2 + (unsigned)j * (8 * BK * 2), w_off[j], uo);
+        const int run = i >> 2, jj = i & 3;
+        const bool is_w = run & 1;
+        const int j = (run >> 1) * 4 + jj;
+        if (jj == 0) lds_dma_base(fetch_lds + (unsigned)(s & 1) * DMA_STAGE_BYTES + (is_w ? BM * BK * 2 : 0) + (unsigned)(run >> 1) * (32 * BK * 2));
+        const u32x4& rsrc = is_w ? w_rsrc : a_rsrc;
+        const unsigned off = is_w ? w_off[j] : a_off[j];
+        if (jj == 0) load_to_lds_16_at<0>(rsrc, off, uo);
+        if (jj == 1) load_to_lds_16_at<1024>(rsrc, off, uo);
+        if (jj == 2) load_to_lds_16_at<2048>(rsrc, off, uo);
+        if (jj == 3) load_to_lds_16_at<3072>(rsrc, off, uo);
     };
     auto fetch_slab = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
