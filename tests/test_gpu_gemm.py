@@ -354,20 +354,22 @@ def test_many_tile_problem_runs_the_256_tile_builds(ctx, build, c_dtype, a32):
     assert np.abs(got[-1] - want[-1]).max() < tol and np.abs(got[:, -1] - want[:, -1]).max() < tol
 
 
+@pytest.mark.parametrize("wdt", [hip.W_BF16, hip.W_F16])
 @pytest.mark.parametrize("k", [64, 192, 320])
-def test_four_wave_build_with_one_three_and_five_slabs(ctx, k):
+def test_four_wave_build_with_one_three_and_five_slabs(ctx, k, wdt):
     # the four-wave loop takes two slabs per trip and requests slabs two ahead: one slab (no
-    # trip, the odd tail only), three and five (trips plus the tail), 169 tiles each
+    # trip, the odd tail only), three and five (trips plus the tail), 169 tiles each; bf16 and
+    # f16 operands (the two MFMA instructions of that build)
     rng = np.random.default_rng(31 + k)
     m, n = 3300, 3290
     a = rng.standard_normal((m, k), dtype=np.float32)
     w = rng.standard_normal((n, k), dtype=np.float32) * np.float32(k ** -0.5)
-    a_bits, ar = to16(a, hip.W_BF16)
-    w_bits, wr = to16(w, hip.W_BF16)
-    raw = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, hip.F32)
+    a_bits, ar = to16(a, wdt)
+    w_bits, wr = to16(w, wdt)
+    raw = run_ext(ctx, a_bits, w_bits, m, k, n, wdt, act_dtype(wdt), hip.F32)
     got = raw.view(np.float32).reshape(m, n)
     check(got, zo.linear_batch(ar, wr), zo.linear_batch(a, w), k, a, w, f"k = {k}")
-    again = run_ext(ctx, a_bits, w_bits, m, k, n, hip.W_BF16, hip.BF16, hip.F32)
+    again = run_ext(ctx, a_bits, w_bits, m, k, n, wdt, act_dtype(wdt), hip.F32)
     assert np.array_equal(raw, again)
 
 
