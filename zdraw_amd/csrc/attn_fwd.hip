@@ -115,6 +115,14 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // conflicts are avoided by swizzling the 16-byte chunk position instead:
     // K chunk c of row r sits at c ^ (r & 15), V chunk c of row r at c ^ ((r & 3) << 2).
     constexpr bool DMA = kDirectLds && std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && NW == 8 && QB == 1;
+    // The product O^T += V^T P^T on v_mfma_f32_16x16x32 (the scores keep the 32 x 32 x 16 form, in
+    // which a lane owns one query). The 16 x 16 form moves half the accumulator bytes per FLOP
+    // through the register file, and at the board's power limit that is worth clock: -2 % of the
+    // kernel's time. It costs a few registers (the compiler writes these MFMAs' results to other
+    // registers than their inputs) and four lane exchanges per block, so only the builds with
+    // room take it: prepared operands, bounded scores. (Giving the scores that form too would
+    // double the MFMA instructions on a vector issue port that the softmax already half fills.)
+    constexpr bool PV16 = DMA && BOUNDED;
     constexpr int KSTAGE = DMA ? KB * D : KS_ELEMS; // elements per ring stage
     constexpr int VSTAGE = DMA ? KB * D : VS_ELEMS;
     // a block enters the ring AHEAD steps before S needs its K (direct loads: one more step, to land)
@@ -377,7 +385,9 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // re-read the last row (they are masked before the softmax).
     const int dma_row = 4 * wave + (lane >> 4);
     const unsigned dma_k_chunk = (unsigned)(((lane & 15) ^ (dma_row & 15)) * 8);
-    const unsigned dma_v_chunk = (unsigned)(((lane & 15) ^ ((dma_row & 3) << 2)) * 8);
+    // (PV16: a row's 16-dim halves also swap with bit 4 of the row, so that the lane groups that
+    // read rows 16 apart hit different banks)
+    const unsigned dma_v_chunk = (unsigned)(((lane & 15) ^ ((dma_row & 3) << 2) ^ (PV16 ? (((dma_row >> 4) & 1) << 1) : 0)) * 8);
     const unsigned dma_k_off = ((unsigned)dma_row * (unsigned)a.k_ts + dma_k_chunk) * 2u;
     const unsigned dma_v_off = ((unsigned)dma_row * (unsigned)a.v_ts + dma_v_chunk) * 2u;
     const int dma_tail_row = min(dma_row, last_row - last_blk * KB);
@@ -411,6 +421,16 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         for (int blk = 0; blk < 4; blk++)
 #pragma unroll
             for (int j = 0; j < 16; j++) oacc[qi][blk][j] = 0.f;
+    // PV16: O^T as 8 x 2 tiles of 16 x 16: with c16 = lane % 16 and g4 = lane / 16 the lane holds query
+    // 16 r + c16, dims 16 dt + 4 g4 + j of tile oacc16[dt][r] (and oacc above stays unused)
+    static_assert(!PV16 || QB == 1, "the 16 x 16 product is written for one 32-query block per wave");
+    const int c16 = lane & 15;
+    const int g4 = lane >> 4;
+    f32x4 oacc16[8][2];
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++)
+#pragma unroll
+        for (int r = 0; r < 2; r++) oacc16[dt][r] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run[QB], l_run[QB]; // running maximum (already multiplied by scale_log2) and denominator half
 #pragma unroll
     for (int qi = 0; qi < QB; qi++) {
@@ -448,6 +468,18 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
         const int col = (DMA ? ((blk ^ tr_row) * 32) : (32 * blk)) + tr_col; // (4 h + tr_row) & 3 == tr_row
         vfo[blk] = lds_address(Vs) + (unsigned)(((4 * h + tr_row) * VROW + col) * 2);
     }
+    // PV16: the patch for output tile dt = 2 blk + x: the 16 lanes of group g4 take keys vkey0 + 8
+    // half + tr_row (vkey0 = 0, 16, 4, 20: the keys whose probabilities the group holds as the
+    // product's B operand, see the exchange in valu_slice), dims 16 dt .. + 15
+    const int vkey0 = 16 * (g4 & 1) + 4 * (g4 >> 1);
+    unsigned vfo16[4][2];
+#pragma unroll
+    for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+        for (int x = 0; x < 2; x++) {
+            const int col = (blk ^ tr_row) * 32 + (x ^ (g4 & 1)) * 16 + 4 * (lane & 3); // (vkey0 + tr_row) & 3 == tr_row
+            vfo16[blk][x] = lds_address(Vs) + (unsigned)(((vkey0 + tr_row) * VROW + col) * 2);
+        }
     typedef const __attribute__((address_space(3))) bf16x8* lds_bf16x8_t;
     typedef __attribute__((address_space(3))) s16x4* lds_s16x4_t;
     auto k_frag = [&](int stage, int s) __attribute__((always_inline)) -> bf16x8 {
@@ -456,6 +488,11 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     auto v_frag = [&](int stage, int kb, int blk, int half) __attribute__((always_inline)) -> s16x4 {
         return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (lds_s16x4_t)(vfo[blk] + (unsigned)(stage * (VSTAGE * 2) + (16 * kb + 8 * half) * (VROW * 2))));
+    };
+
+    auto v_frag16 = [&](int stage, int dt, int half) __attribute__((always_inline)) -> s16x4 {
+        return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_s16x4_t)(vfo16[dt >> 1][dt & 1] + (unsigned)(stage * (VSTAGE * 2) + (8 * half) * (VROW * 2))));
     };
 
     // S^T block = K(block) . Q^T for both query blocks
@@ -475,6 +512,19 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 
     // O^T += V(block)^T . P^T
     auto pv_block = [&](int stage, const bf16x8 (&p)[QB][2]) {
+        if constexpr (PV16) { // p[0][r] is the B operand of query tile r
+#pragma unroll
+            for (int dt = 0; dt < 8; dt++) {
+                const s16x4 lo = v_frag16(stage, dt, 0);
+                const s16x4 hi = v_frag16(stage, dt, 1);
+                typedef short s16x8 __attribute__((ext_vector_type(8)));
+                const bf16x8 vf = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+                for (int r = 0; r < 2; r++)
+                    oacc16[dt][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p[0][r], oacc16[dt][r], 0, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
@@ -502,8 +552,13 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     auto frag_read = [&](int k_stage, int v_stage, int slot) __attribute__((always_inline)) {
         if (slot & 1) {
             const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
-            vlo[idx] = v_frag(v_stage, kb, blk, 0);
-            vhi[idx] = v_frag(v_stage, kb, blk, 1);
+            if constexpr (PV16) { // the two patches of output tile idx
+                vlo[idx] = v_frag16(v_stage, idx, 0);
+                vhi[idx] = v_frag16(v_stage, idx, 1);
+            } else {
+                vlo[idx] = v_frag(v_stage, kb, blk, 0);
+                vhi[idx] = v_frag(v_stage, kb, blk, 1);
+            }
         } else {
             kf[slot >> 1] = k_frag(k_stage, slot >> 1);
         }
@@ -538,7 +593,14 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
             for (int i = 0; i < 8; i++) pin(kfo[i]);
 #pragma unroll
-            for (int i = 0; i < 4; i++) pin(vfo[i]);
+            for (int i = 0; i < 4; i++) {
+                if constexpr (PV16) {
+                    pin(vfo16[i][0]);
+                    pin(vfo16[i][1]);
+                } else {
+                    pin(vfo[i]);
+                }
+            }
         }
 #ifdef HACK16
         auto mfma_half = [&](int slot, int part) __attribute__((always_inline)) {
@@ -567,9 +629,15 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
                 const bf16x8 vf =
                     __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(vlo[idx], vhi[idx], 0, 1, 2, 3, 4, 5, 6, 7));
+                if constexpr (PV16) {
 #pragma unroll
-                for (int qi = 0; qi < QB; qi++)
-                    oacc[qi][blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_prev[qi][kb], oacc[qi][blk], 0, 0, 0);
+                    for (int r = 0; r < 2; r++)
+                        oacc16[idx][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_prev[0][r], oacc16[idx][r], 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int qi = 0; qi < QB; qi++)
+                        oacc[qi][blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p_prev[qi][kb], oacc[qi][blk], 0, 0, 0);
+                }
             } else {
                 const int st = slot >> 1;
 #pragma unroll
@@ -601,6 +669,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 
         float mc[QB], alpha[QB], psum[QB];
         unsigned pc[QB][8] = {}; // P as packed bf16 pairs
+        u32x4 pb[2] = {};        // PV16: the same after the exchange between lane rows
 #pragma unroll
         for (int qi = 0; qi < QB; qi++) {
             mc[qi] = (!BOUNDED && !REFACC && m_run[qi] != -INFINITY) ? m_run[qi] : 0.f;
@@ -643,7 +712,25 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                     // watch after the slots adds the denominator
                     if ((c & 1) == 0) exp_pair(qi, c >> 1, std::integral_constant<bool, !REFACC>{});
                 }
-                if (c == 15) {
+                if constexpr (PV16) {
+                    // The exponentiated block as the product's B operands. pc[k] packs this lane's
+                    // scores 2 k and 2 k + 1 of its query (keys 8 (k / 2) + 4 h + 2 (k % 2) .. + 1).
+                    // v_permlane16_swap of pc[k] and pc[k + 4] returns [a.row0, b.row0, a.row2, b.row2]
+                    // and [a.row1, b.row1, a.row3, b.row3] (rows of 16 lanes): the first holds queries
+                    // 0..15 on every lane row, the second queries 16..31, and lane row g4 holds keys
+                    // vkey0 + {0..3, 8..11}: eight of the block's 32 keys per group, as the 16 x 16 x
+                    // 32 MFMA's B operand wants them. One pair per odd slice, as soon as both exist.
+                    if (c >= 9 && (c & 1)) {
+                        const int k = (c - 9) >> 1;
+                        const u32x2 r = __builtin_amdgcn_permlane16_swap(pc[qi][k], pc[qi][k + 4], false, false);
+                        pb[0][k] = r[0];
+                        pb[1][k] = r[1];
+                    }
+                    if (c == 15) {
+                        p_cur[qi][0] = __builtin_bit_cast(bf16x8, pb[0]);
+                        p_cur[qi][1] = __builtin_bit_cast(bf16x8, pb[1]);
+                    }
+                } else if (c == 15) {
                     p_cur[qi][0] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][0], pc[qi][1], pc[qi][2], pc[qi][3]});
                     p_cur[qi][1] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][4], pc[qi][5], pc[qi][6], pc[qi][7]});
                 }
@@ -889,31 +976,116 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     }
 
     // ---- epilogue: O = O^T / l
-#pragma unroll
-    for (int qi = 0; qi < QB; qi++) {
-        const float l_tot = pair_sum(l_run[qi]);
+    if constexpr (PV16) {
+        // The denominator lives with the scores (lane = query l32); the lane that holds query
+        // 16 r + c16 of O^T fetches it from there.
+        const float l_tot = pair_sum(l_run[0]);
         const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-        const int qrow = q0 + 32 * qi + l32;
+        float inv_r[2];
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+            inv_r[r] = __uint_as_float((unsigned)__builtin_amdgcn_ds_bpermute(4 * (16 * r + c16), (int)__float_as_uint(inv_l)));
         if (a.splits > 1) {
             // unnormalised rows, reference point and denominator of this part
-            const int64_t prow = ((int64_t)blockIdx.x * BQ + wave * QR + 32 * qi + l32);
-            float* op = a.part_o + prow * D;
+            const int64_t prow0 = (int64_t)blockIdx.x * BQ + wave * QR;
 #pragma unroll
-            for (int blk = 0; blk < 4; blk++)
+            for (int r = 0; r < 2; r++) {
+                float* op = a.part_o + (prow0 + 16 * r + c16) * D + 4 * g4;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    f32x4 v;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j];
-                    *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
-                }
+                for (int dt = 0; dt < 8; dt++) *reinterpret_cast<f32x4*>(op + 16 * dt) = oacc16[dt][r];
+            }
             if (h == 0) {
-                a.part_ml[prow * 2] = BOUNDED ? 0.f : m_run[qi];
-                a.part_ml[prow * 2 + 1] = l_tot;
+                a.part_ml[(prow0 + l32) * 2] = BOUNDED ? 0.f : m_run[0];
+                a.part_ml[(prow0 + l32) * 2 + 1] = l_tot;
             }
         } else if (a.out_dtype == kF32) {
-            if (qrow < a.tokens) {
-                float* op = reinterpret_cast<float*>(a.o) + (int64_t)seg * a.o_bs + (int64_t)qrow * a.o_ts + (int64_t)head * a.o_hs;
+#pragma unroll
+            for (int r = 0; r < 2; r++) {
+                const int qrow = q0 + 16 * r + c16;
+                if (qrow < a.tokens) {
+                    float* op = reinterpret_cast<float*>(a.o) + (int64_t)seg * a.o_bs + (int64_t)qrow * a.o_ts + (int64_t)head * a.o_hs + 4 * g4;
+#pragma unroll
+                    for (int dt = 0; dt < 8; dt++) *reinterpret_cast<f32x4*>(op + 16 * dt) = oacc16[dt][r] * inv_r[r];
+                }
+            }
+        } else {
+            // 16-bit output: a lane holds 8-byte pieces of two rows, which would leave the chip as
+            // 16 thirty-two-byte segments per store instruction. The wave turns its 32 x 128 tile
+            // through 8 KB of LDS (its own stage of the idle K ring, K layout: chunk c of row r
+            // at c ^ (r & 15)) and stores whole 256-byte rows, four per instruction.
+            __syncthreads(); // every wave is done with the ring
+            typedef __attribute__((address_space(3))) u32x2* lds_u32x2_t;
+            typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
+            typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+            const unsigned o_lds = lds_address(Ks) + (unsigned)(wave * (KSTAGE * 2));
+            const bool half = a.out_dtype == kF16;
+#pragma unroll
+            for (int r = 0; r < 2; r++)
+#pragma unroll
+                for (int dt = 0; dt < 8; dt++) {
+                    // row 16 r + c16, dims 16 dt + 4 g4 .. + 3: chunk 2 dt + g4 / 2, half g4 % 2
+                    const f32x4 v = oacc16[dt][r] * inv_r[r];
+                    const u32x2 bits = half ? __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4))
+                                            : __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
+                    *(lds_u32x2_t)(o_lds + (unsigned)((16 * r + c16) * (D * 2) + (((2 * dt + (g4 >> 1)) ^ c16) * 16) + 8 * (g4 & 1))) = bits;
+                }
+            unsigned short* const obase = reinterpret_cast<unsigned short*>(a.o) + (int64_t)seg * a.o_bs + (int64_t)head * a.o_hs;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int r = 4 * j + (lane >> 4);
+                const u32x4 row16 = *(lds_u32x4_t)(o_lds + (unsigned)(r * (D * 2) + (lane & 15) * 16));
+                const int orow = q0 + r;
+                if (orow < a.tokens)
+                    *reinterpret_cast<u32x4*>(obase + (int64_t)orow * a.o_ts + (((lane & 15) ^ (r & 15)) * 8)) = row16;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int qi = 0; qi < QB; qi++) {
+            const float l_tot = pair_sum(l_run[qi]);
+            const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+            const int qrow = q0 + 32 * qi + l32;
+            if (a.splits > 1) {
+                // unnormalised rows, reference point and denominator of this part
+                const int64_t prow = ((int64_t)blockIdx.x * BQ + wave * QR + 32 * qi + l32);
+                float* op = a.part_o + prow * D;
+#pragma unroll
+                for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        f32x4 v;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j];
+                        *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
+                    }
+                if (h == 0) {
+                    a.part_ml[prow * 2] = BOUNDED ? 0.f : m_run[qi];
+                    a.part_ml[prow * 2 + 1] = l_tot;
+                }
+            } else if (a.out_dtype == kF32) {
+                if (qrow < a.tokens) {
+                    float* op = reinterpret_cast<float*>(a.o) + (int64_t)seg * a.o_bs + (int64_t)qrow * a.o_ts + (int64_t)head * a.o_hs;
+#pragma unroll
+                    for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            f32x4 v;
+#pragma unroll
+                            for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
+                            *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
+                        }
+                }
+            } else {
+                // 16-bit output: a lane holds one row in 8-byte pieces, which would leave the chip as
+                // 32 sixteen-byte segments per store instruction. The wave turns its 32 x 128 tile
+                // through 8 KB of LDS (its own stage of the idle K ring, K layout: chunk c of row r
+                // at c ^ (r & 15)) and stores whole 256-byte rows, four per instruction.
+                __syncthreads(); // every wave is done with the ring
+                typedef __attribute__((address_space(3))) u32x2* lds_u32x2_t;
+                typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
+                typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+                const unsigned o_lds = lds_address(Ks) + (unsigned)((wave * QB + qi) * (KSTAGE * 2));
+                const bool half = a.out_dtype == kF16;
 #pragma unroll
                 for (int blk = 0; blk < 4; blk++)
 #pragma unroll
@@ -921,39 +1093,19 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                         f32x4 v;
 #pragma unroll
                         for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
-                        *reinterpret_cast<f32x4*>(op + 32 * blk + 8 * i + 4 * h) = v;
+                        const u32x2 bits = half ? __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4))
+                                                : __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
+                        *(lds_u32x2_t)(o_lds + (unsigned)(l32 * (D * 2) + (((4 * blk + i) ^ (l32 & 15)) * 16) + 8 * h)) = bits;
                     }
-            }
-        } else {
-            // 16-bit output: a lane holds one row in 8-byte pieces, which would leave the chip as
-            // 32 sixteen-byte segments per store instruction. The wave turns its 32 x 128 tile
-            // through 8 KB of LDS (its own stage of the idle K ring, K layout: chunk c of row r
-            // at c ^ (r & 15)) and stores whole 256-byte rows, four per instruction.
-            __syncthreads(); // every wave is done with the ring
-            typedef __attribute__((address_space(3))) u32x2* lds_u32x2_t;
-            typedef const __attribute__((address_space(3))) u32x4* lds_u32x4_t;
-            typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-            const unsigned o_lds = lds_address(Ks) + (unsigned)((wave * QB + qi) * (KSTAGE * 2));
-            const bool half = a.out_dtype == kF16;
+                unsigned short* const obase = reinterpret_cast<unsigned short*>(a.o) + (int64_t)seg * a.o_bs + (int64_t)head * a.o_hs;
 #pragma unroll
-            for (int blk = 0; blk < 4; blk++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    f32x4 v;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) v[j] = oacc[qi][blk][4 * i + j] * inv_l;
-                    const u32x2 bits = half ? __builtin_bit_cast(u32x2, __builtin_convertvector(v, f16x4))
-                                            : __builtin_bit_cast(u32x2, __builtin_convertvector(v, bf16x4));
-                    *(lds_u32x2_t)(o_lds + (unsigned)(l32 * (D * 2) + (((4 * blk + i) ^ (l32 & 15)) * 16) + 8 * h)) = bits;
+                for (int j = 0; j < 8; j++) {
+                    const int r = 4 * j + (lane >> 4);
+                    const u32x4 row16 = *(lds_u32x4_t)(o_lds + (unsigned)(r * (D * 2) + (lane & 15) * 16));
+                    const int orow = q0 + 32 * qi + r;
+                    if (orow < a.tokens)
+                        *reinterpret_cast<u32x4*>(obase + (int64_t)orow * a.o_ts + (((lane & 15) ^ (r & 15)) * 8)) = row16;
                 }
-            unsigned short* const obase = reinterpret_cast<unsigned short*>(a.o) + (int64_t)seg * a.o_bs + (int64_t)head * a.o_hs;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int r = 4 * j + (lane >> 4);
-                const u32x4 row16 = *(lds_u32x4_t)(o_lds + (unsigned)(r * (D * 2) + (lane & 15) * 16));
-                const int orow = q0 + 32 * qi + r;
-                if (orow < a.tokens)
-                    *reinterpret_cast<u32x4*>(obase + (int64_t)orow * a.o_ts + (((lane & 15) ^ (r & 15)) * 8)) = row16;
             }
         }
     }
