@@ -120,9 +120,10 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // through the register file, and at the board's power limit that is worth clock: -2 % of the
     // kernel's time. It costs a few registers (the compiler writes these MFMAs' results to other
     // registers than their inputs) and four lane exchanges per block, so only the builds with
-    // room take it: prepared operands, bounded scores. (Giving the scores that form too would
-    // double the MFMA instructions on a vector issue port that the softmax already half fills.)
-    constexpr bool PV16 = DMA && BOUNDED;
+    // room take it: prepared operands, and not the running maximum together with a mask (that
+    // build then spills inside the loop). (Giving the scores that form too would double the MFMA
+    // instructions on a vector issue port that the softmax already half fills.)
+    constexpr bool PV16 = DMA && (BOUNDED || !MASKED);
     constexpr int KSTAGE = DMA ? KB * D : KS_ELEMS; // elements per ring stage
     constexpr int VSTAGE = DMA ? KB * D : VS_ELEMS;
     // a block enters the ring AHEAD steps before S needs its K (direct loads: one more step, to land)
@@ -442,13 +443,9 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // relative to the reference and the exponentials need no subtraction.
     // (Only the builds with registers to spare: prepared 16-bit operands. The others subtract.)
     constexpr bool REFACC = !BOUNDED && KMODE == kQkNone && std::is_same<TIn, bf16_t>::value && NW == 8 && QB == 1;
-    f32x16 negm[REFACC ? QB : 1];
-    if constexpr (REFACC) {
+    float negm[QB]; // (one value per lane: every element of the accumulator starts from it)
 #pragma unroll
-        for (int qi = 0; qi < QB; qi++)
-#pragma unroll
-            for (int j = 0; j < 16; j++) negm[qi][j] = 0.f;
-    }
+    for (int qi = 0; qi < QB; qi++) negm[qi] = 0.f;
 
     // LDS byte addresses of this lane's fragments in ring stage 0; a stage, a key half (kb)
     // and a row half add constants. K: key row l32, dims 16 s + 8 h .. +7 (8 addresses, the
@@ -665,7 +662,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
         for (int qi = 0; qi < QB; qi++)
 #pragma unroll
-            for (int j = 0; j < 16; j++) s_next[qi][j] = REFACC ? negm[qi][j] : 0.f;
+            for (int j = 0; j < 16; j++) s_next[qi][j] = REFACC ? negm[qi] : 0.f;
 
         float mc[QB], alpha[QB], psum[QB];
         unsigned pc[QB][8] = {}; // P as packed bf16 pairs
@@ -832,16 +829,38 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
                         for (int j = 0; j < 16; j++) {
                             s_next[qi][j] -= mc[qi];
-                            negm[qi][j] = -ref_new;
+                            negm[qi] = -ref_new;
                         }
                     }
                     l_run[qi] *= alpha[qi];
+                    if constexpr (PV16) {
+                        // O^T holds other queries on this lane than the scores do: the factor of
+                        // query 16 r + c16 comes from the lane that owns that query's scores
 #pragma unroll
-                    for (int blk = 0; blk < 4; blk++)
+                        for (int r = 0; r < 2; r++) {
+                            const float ar = __uint_as_float((unsigned)__builtin_amdgcn_ds_bpermute(4 * (16 * r + c16), (int)__float_as_uint(alpha[qi])));
 #pragma unroll
-                        for (int j = 0; j < 16; j++) oacc[qi][blk][j] *= alpha[qi];
-                    p_cur[qi][0] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][0], pc[qi][1], pc[qi][2], pc[qi][3]});
-                    p_cur[qi][1] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][4], pc[qi][5], pc[qi][6], pc[qi][7]});
+                            for (int dt = 0; dt < 8; dt++) oacc16[dt][r] *= ar;
+                        }
+                    } else {
+#pragma unroll
+                        for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+                            for (int j = 0; j < 16; j++) oacc[qi][blk][j] *= alpha[qi];
+                    }
+                    if constexpr (PV16) { // the exchange of valu_slice, on the pairs taken again
+#pragma unroll
+                        for (int k = 0; k < 4; k++) {
+                            const u32x2 r = __builtin_amdgcn_permlane16_swap(pc[qi][k], pc[qi][k + 4], false, false);
+                            pb[0][k] = r[0];
+                            pb[1][k] = r[1];
+                        }
+                        p_cur[qi][0] = __builtin_bit_cast(bf16x8, pb[0]);
+                        p_cur[qi][1] = __builtin_bit_cast(bf16x8, pb[1]);
+                    } else {
+                        p_cur[qi][0] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][0], pc[qi][1], pc[qi][2], pc[qi][3]});
+                        p_cur[qi][1] = __builtin_bit_cast(bf16x8, u32x4{pc[qi][4], pc[qi][5], pc[qi][6], pc[qi][7]});
+                    }
                 }
             }
 #pragma unroll
