@@ -39,6 +39,7 @@ namespace fwd {
 
 // Schedule constants of the pipelined step (the measured best of what was tried).
 constexpr int kLdsLookahead = 4;   // slots between an LDS fragment read and the MFMA that consumes it
+constexpr int kLdsLookaheadDirect = 6; // the same for the direct-to-LDS build (8 is 0.3 % better still where it does not spill)
 constexpr int kReadBatch = 2;      // slots whose fragment reads are issued together (one wait per batch)
 constexpr int kMfmaPrio = 1;       // wave priority while an MFMA is issued, builds that stage blocks through registers (0 = leave it alone)
 constexpr int kMfmaPrioDirect = 0; // the same for the direct-to-LDS build
@@ -128,7 +129,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     constexpr int VSTAGE = DMA ? KB * D : VS_ELEMS;
     // a block enters the ring AHEAD steps before S needs its K (direct loads: one more step, to land)
     constexpr int AHEAD = NST == 8 ? (DMA ? 5 : 4) : 2;
-    constexpr int LA = kLdsLookahead;   // slots between an LDS fragment read and its MFMA
+    constexpr int LA = DMA ? kLdsLookaheadDirect : kLdsLookahead; // slots between an LDS fragment read and its MFMA
     constexpr int RB = kReadBatch;      // slots whose reads are issued together (divides 16 and LA)
     // Wave priority while an MFMA is being issued. The register-staged builds gain from it (the
     // masked one loses 13 % without). The direct-to-LDS build runs 5 % fewer cycles per
