@@ -57,6 +57,24 @@ def cpu_baseline(w, seconds_target=15.0):
     }
 
 
+class ContextOnCus:
+    """The host context with its queue swapped for one confined to `cu_count` compute units
+    (zdraw_hip_create_queue_on_cus, a measurement aid): `--cu-count`."""
+
+    def __init__(self, L, ctx, cu_count):
+        self._L, self._ctx = L, ctx
+        self.queue = L.zdraw_hip_create_queue_on_cus(ctx.device, cu_count)
+        if not self.queue:
+            raise RuntimeError("zdraw_hip_create_queue_on_cus failed")
+
+    def __getattr__(self, name):
+        return getattr(self._ctx, name)
+
+    def deinit(self):
+        self._L.zdraw_hip_release_queue(self.queue)
+        self._ctx.deinit()
+
+
 def timed_region(L, ctx, res, steps):
     """K launches back to back on the library's stream, bracketed by a full
     synchronisation on both sides (wall clock); the attention kernel of every
@@ -472,7 +490,7 @@ def main():
     ap.add_argument("--no-side-legs", action="store_true",
                     help="skip the short untimed-by-value legs (other softmax form, other benchmark shapes, the GEMM, chain and wide-head paths)")
     ap.add_argument("--cu-count", type=int, default=0,
-                    help="confine the library's stream to this many compute units (0 = all): shows whether "
+                    help="(attention path) confine the stream to this many compute units (0 = all): shows whether "
                          "the kernel's time follows the CU count or the board's power limit")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a known-size kernel to scale "
@@ -480,8 +498,6 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)")
-    if args.cu_count > 0:
-        os.environ["ZDRAW_HIP_CU_COUNT"] = str(args.cu_count)  # read when the library creates its stream
     if args.path in PATH_MAINS:
         print(json.dumps(PATH_MAINS[args.path](args)), flush=True)
         return
@@ -494,6 +510,8 @@ def main():
 
     L = hip.lib()
     ctx = host.Context.init()
+    if args.cu_count > 0:
+        ctx = ContextOnCus(L, ctx, args.cu_count)
     L.zdraw_hip_set_attention_variant(args.variant)
     w = wl.by_name(args.workload, seed=0)
     k_site = hip.K_PREPASS if args.k_site == "prepass" else hip.K_IN_TILE_LOAD

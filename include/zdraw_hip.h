@@ -102,11 +102,21 @@ typedef struct ZdrawHipAttnExt {
      * lets the kernel exponentiate scores without tracking a running maximum
      * (softmax is shift-invariant); 0 or a larger bound selects the running-maximum
      * form. When the call carries norm weights (qk_mode != NONE) the library forms
-     * sqrt(head_dim) * max|w_q| * max|w_k| from the weight buffers itself (read once
-     * per buffer, until the buffer is written or released) and decides on the larger of
-     * the two values: the caller's figure can only make the choice more cautious, a figure
-     * that is too small cannot overflow. With qk_mode NONE there are no weights to check
-     * and the caller's figure stands. */
+     * sqrt(head_dim) * max|w_q| * max|w_k| from the weight buffers itself and decides on
+     * the larger of the two values: the caller's figure can only make the choice more
+     * cautious, a figure that is too small cannot overflow. It does so only for weight
+     * buffers whose bytes cannot change behind its back: memory the library allocated
+     * (create_buffer, _with_data, _no_copy), whose device address was never handed out
+     * (buffer_device_ptr) and which no kernel of this library was ever asked to write;
+     * their 128 weights are read back once and the figure kept until write_buffer or
+     * release. With any other weight buffer (wrap_device_memory, an exposed or
+     * kernel-written buffer) the call takes the running-maximum form whatever the
+     * caller's figure says. With qk_mode NONE there are no weights to check and the
+     * caller's figure stands.
+     * Accuracy: Q' and K' are rounded to 16 bits before the product, so a score of s
+     * nats carries an absolute error of about s * 2^-8 (bf16 operands) or s * 2^-11
+     * (ZDRAW_HIP_F16 staging, see `staging`); scores reach sqrt(head_dim) * max|w_q| *
+     * max|w_k| = 11.3 nats with unit weights and grow with the product of the weights. */
     float score_bound;
     uint32_t reserved;
 } ZdrawHipAttnExt;
@@ -136,15 +146,37 @@ void zdraw_hip_release_queue(void* queue);
 /* ---- buffers (metal_c.zig:12-33) ----------------------------------------- */
 void* zdraw_hip_create_buffer(void* device, size_t size);
 void* zdraw_hip_create_buffer_with_data(void* device, const uint8_t* data, size_t size);
-/* Borrowed DEVICE memory (e.g. a tensor another runtime owns): never freed by
- * release_buffer. The Metal call wraps host memory; on a discrete GPU the
- * no-copy form only makes sense for memory already on the device. */
-void* zdraw_hip_create_buffer_no_copy(void* device, void* device_ptr, size_t size);
+/* metal_c.zig:18-22, metal_api.m:601-638: a buffer over `size` bytes of HOST memory that the
+ * caller keeps owning (mbuffer.Cache.trySliceBind / sourceBuffer hand it a slice of the mmapped
+ * checkpoint, metal/mbuffer.zig:88, 129). Unified memory lets Metal wrap those pages; a discrete
+ * GPU cannot read them at speed, so the bytes are uploaded once here, when the buffer is
+ * created (the sources are immutable weights), and the kernels read the device copy. Any
+ * address and length is accepted (the Metal call returns NULL for a pointer that is not
+ * page-aligned and its caller then binds the whole mapping at an offset: both bindings work
+ * here). `data` is not read again after the call returns; release_buffer /
+ * release_weight_buffer free the device copy only. NULL when the allocation or upload fails. */
+void* zdraw_hip_create_buffer_no_copy(void* device, const uint8_t* data, size_t size);
+/* No counterpart in the reference (interop with memory another runtime already holds on the
+ * GPU, e.g. a tensor): a buffer handle over `size` bytes of DEVICE memory at device_ptr, never
+ * freed by release_buffer. The pointer is checked with the runtime (hipPointerGetAttributes,
+ * hipMemGetAddressRange): NULL unless [device_ptr, device_ptr + size) lies inside one device
+ * allocation on this device, so host memory cannot reach a kernel through this call. The
+ * library never caches anything it read from such memory (see score_bound above). */
+void* zdraw_hip_wrap_device_memory(void* device, void* device_ptr, size_t size);
 void zdraw_hip_read_buffer(void* buffer, uint8_t* dst, size_t size);
+/* metal_c.zig:24-29, metal_api.m:647-665: the readback that works for every buffer and is
+ * ordered after the work enqueued on `queue` (waits for the queue, then copies).
+ * 0, -1 for a null or short buffer, -2 when the device reports an error. */
+int zdraw_hip_read_buffer_any(void* queue, void* buffer, uint8_t* dst, size_t size);
 void zdraw_hip_write_buffer(void* buffer, const uint8_t* src, size_t size);
 size_t zdraw_hip_buffer_length(void* buffer);
-void* zdraw_hip_buffer_device_ptr(void* buffer); /* no reference counterpart: interop */
+/* No reference counterpart: interop. A buffer whose device address has been handed out may
+ * change behind the library's back; from then on nothing read from it is cached. */
+void* zdraw_hip_buffer_device_ptr(void* buffer);
 void zdraw_hip_release_buffer(void* buffer);
+/* metal_c.zig:32, metal_api.m:686-692: release of a buffer made by create_buffer_no_copy (the
+ * reference keeps a separate weight-footprint ledger); the same as release_buffer here. */
+void zdraw_hip_release_weight_buffer(void* buffer);
 
 /* ---- pipelines (metal_c.zig:99-107) -------------------------------------- */
 /* Same argument list as zdraw_metal_compile (metal_c.zig:99-105). The kernels are
@@ -221,12 +253,16 @@ int zdraw_hip_run_qk_norm_rope_ext(void* queue, void* pipeline, void* q, void* k
 /* metal_c.zig:148-159 with QkNormParams (metal_c.zig:258-274), argument for argument: the
  * Z-Image qk_norm_rope dispatch behind mqk.run (metal/mqk.zig:20-58). In place on f32
  * token-major q [tokens][heads][head_dim] and k [tokens][kv_heads][head_dim]; q_weight /
- * k_weight hold head_dim norm weights of type params->q_dtype / k_dtype at byte offsets
- * params->q_offset / k_offset; pos is u64 [tokens][3]; rope the (cos,sin) f32 pair table
- * (zrope.Cache.pairBytes) whose axes start at params->base0..2 pairs. thread_count is
- * accepted and not used. A position past its axis (zimage/zrope.zig:48 refuses those on the
- * host) reads the axis's last table entry instead of memory outside the table. Blocks until
- * done; returns 0, or 1 / 2 / negative as above. */
+ * k_weight hold head_dim norm weights of type params->q_dtype / k_dtype (each f16, bf16 or
+ * f32, independently) at byte offsets params->q_offset / k_offset, which need only be
+ * multiples of the element size (mbuffer.Cache.bindView hands over file offsets,
+ * metal/mqk.zig:97-98); weights of two types or off a 16-byte boundary are first copied as
+ * f32 into 1 KiB of the queue's scratch by a small launch. pos is u64 [tokens][3]; rope the
+ * (cos,sin) f32 pair table (zrope.Cache.pairBytes) whose axes start at params->base0..2
+ * pairs. thread_count is accepted and not used. A position past its axis
+ * (zimage/zrope.zig:48 refuses those on the host) reads the axis's last table entry
+ * instead of memory outside the table. Blocks until done; returns 0, or 1 / 2 / negative
+ * as above. */
 typedef struct ZdrawQkNormParams { /* metal_c.zig:258-274, 80 bytes */
     uint32_t tokens, heads, kv_heads, head_dim;
     uint32_t q_dtype, k_dtype; /* element type of q_norm / k_norm: 1 f16, 2 bf16, 3 f32 */

@@ -6,12 +6,7 @@
  * between builds of one kernel and to read the shader clock a launch really ran at. They
  * change process-wide state and are not part of the drop-in boundary (include/zdraw_hip.h).
  *
- * Environment read by zdraw_hip_create_device / zdraw_hip_create_queue, also measurement only:
- *   ZDRAW_ATTN_VARIANT = n   as zdraw_hip_set_attention_variant(n)
- *   ZDRAW_GEMM_BUILD = n     as zdraw_hip_set_gemm_build(n)
- *   ZDRAW_HIP_CU_COUNT = n   the queue's stream is confined to n compute units (0 < n < the
- *                            device's CU count): does a kernel's time follow the CU count or
- *                            the board's power limit
+ * The library itself reads no environment variable for any of this.
  */
 #ifndef ZDRAW_HIP_MEASURE_H
 #define ZDRAW_HIP_MEASURE_H
@@ -34,15 +29,17 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
 /* Which build of the attention kernel runs. Bit 0: 0 = 8 waves x 32 query rows per
  * workgroup, one workgroup per CU (default); 1 = 4 waves x 32 query rows, two workgroups
  * per CU. Bit 1: 2 = never split the tiles of a thinly filled last round along the keys
- * (by default they are). Bit 2: 4 = the role-split build for prepared bf16 operands on the
- * 8-wave shape (the two waves of a SIMD share 64 query rows: one forms the scores and the
- * softmax, the other the product with V; a quarter less LDS traffic per MFMA, more cycles
- * per key block: slower, kept for measurement). */
+ * (by default they are). */
 void zdraw_hip_set_attention_variant(int variant);
 
 /* Which build multiplies 256 x 256 tiles of 16-bit activations. 1 = four waves, 128 x 128
  * each (default); 0 = eight waves, 64 x 128 each. */
 void zdraw_hip_set_gemm_build(int build);
+
+/* A queue as zdraw_hip_create_queue makes it, its stream confined to cu_count compute units
+ * (0 < cu_count < the device's CU count; anything else: an ordinary queue): does a kernel's
+ * time follow the CU count or the board's power limit. */
+void* zdraw_hip_create_queue_on_cus(void* device, int cu_count);
 
 #ifdef __cplusplus
 }

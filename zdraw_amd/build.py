@@ -44,25 +44,31 @@ def build_hip(verbose: bool = False, out: str | None = None, extra_flags=()) -> 
     target = out or HIP_LIB
     tag = "" if out is None else "." + os.path.basename(out)
     srcs = [os.path.join(CSRC, f) for f in ("attn_fwd.hip", "attn_wide.hip", "qk_prepass.hip", "gemm_half.hip", "bridge.hip")]
-    objs = []
-    for src in srcs:
-        obj = os.path.join(LIBDIR, os.path.basename(src) + tag + ".o")
-        _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-c", src, "-o", obj])
-        objs.append(obj)
+    from concurrent.futures import ThreadPoolExecutor
+    objs = [os.path.join(LIBDIR, os.path.basename(src) + tag + ".o") for src in srcs]
+    with ThreadPoolExecutor(max_workers=min(len(srcs), os.cpu_count() or 1)) as pool:  # one hipcc per source file
+        list(pool.map(lambda so: _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-c", so[0], "-o", so[1]]), zip(srcs, objs)))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", target, *objs])
     if verbose:
         print("built", target)
     return target
 
 
+_ASM_CACHE: dict = {}
+
+
 def _device_asm(src: str, extra_flags=()) -> list[str]:
     import tempfile
+    key = (src, tuple(extra_flags), os.path.getmtime(src))
+    if key in _ASM_CACHE:
+        return _ASM_CACHE[key]
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     with tempfile.TemporaryDirectory() as tmp:
         asm = os.path.join(tmp, "out.s")
         _run([hipcc, *HIPCC_FLAGS, *extra_flags, "-S", "--cuda-device-only", "-o", asm, src])
         with open(asm) as f:
-            return f.read().split("\n")
+            _ASM_CACHE[key] = f.read().split("\n")
+    return _ASM_CACHE[key]
 
 
 def m0_writes(src: str = os.path.join(CSRC, "gemm_half.hip"), kernel_substr: str = "gemm_ring_kernel", extra_flags=()) -> list[str]:
@@ -130,9 +136,20 @@ def build_host(verbose: bool = False) -> str:
     return HOST_LIB
 
 
+def check_hand_scheduled_kernels(verbose: bool = False):
+    """The GEMM's hand-placed MFMAs and its M0 held across loads are safe only as long as the
+    compiler puts nothing of its own in between: a toolchain that does fails the build here."""
+    bad = m0_writes() + tied_mfma_hazards()
+    if bad:
+        raise RuntimeError("gemm_half.hip compiled to code that breaks its hand-written schedule:\n  " + "\n  ".join(bad))
+    if verbose:
+        print("hand-scheduled kernels: no foreign M0 write, no accumulator touched inside an MFMA run")
+
+
 def build_all(verbose: bool = False):
     build_hip(verbose)
     build_host(verbose)
+    check_hand_scheduled_kernels(verbose)
 
 
 if __name__ == "__main__":

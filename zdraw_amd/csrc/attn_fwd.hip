@@ -600,27 +600,6 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 }
             }
         }
-#ifdef HACK16
-        auto mfma_half = [&](int slot, int part) __attribute__((always_inline)) {
-            if (slot & 1) {
-                const int idx = slot >> 1, kb = idx >> 2, blk = idx & 3;
-                const bf16x8 vf =
-                    __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(vlo[idx], vhi[idx], 0, 1, 2, 3, 4, 5, 6, 7));
-                f32x16& c = oacc[0][blk];
-                const int q = 2 * kb + part;
-                f32x4 c0 = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
-                c0 = part ? __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_prev[0][kb], vf, c0, 0, 0, 0) : __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_prev[0][kb], c0, 0, 0, 0);
-                for (int j = 0; j < 4; j++) c[4 * q + j] = c0[j];
-            } else {
-                const int st = slot >> 1;
-                f32x16& c = s_next[0];
-                const int q = 2 * (st & 1) + part;
-                f32x4 c0 = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
-                c0 = part ? __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[0][st], kf[st], c0, 0, 0, 0) : __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[st], qf[0][st], c0, 0, 0, 0);
-                for (int j = 0; j < 4; j++) c[4 * q + j] = c0[j];
-            }
-        };
-#endif
         auto mfma_slot = [&](int slot) __attribute__((always_inline)) {
             if (MFMA_PRIO) __builtin_amdgcn_s_setprio(MFMA_PRIO);
             if (slot & 1) {
@@ -751,28 +730,8 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                     else if constexpr (XSTEP) frag_read(stage_of(2), stage_of(0), slot - 16);
                 }
             }
-#if !defined(HACK16)
             mfma_slot(g);
             valu_slice(g);
-#elif HACK16 == 1
-            mfma_half(g, 0);
-            mfma_half(g, 1);
-            valu_slice(g);
-#elif HACK16 == 2
-            mfma_half(g, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            valu_slice(g);
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_half(g, 1);
-#elif HACK16 == 3
-            // the VALU work of an even slot is split over the even slot's second half and the odd slot's first half
-            mfma_half(g, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if ((g & 1) == 0) valu_slice(g);
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_half(g, 1);
-            if (g & 1) valu_slice(g);
-#endif
             // ring: block b+AHEAD (in this register set since two steps ago) goes to its stage,
             // whose previous tenant's last reader (V, NST-AHEAD-1 steps back) is at least one
             // barrier behind; then the set starts loading block b+AHEAD+2
@@ -1135,12 +1094,6 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     }
 }
 
-} // namespace fwd
-} // namespace zdraw
-namespace zdraw {
-namespace fwd {
-#include "attn_pair.hpp"
-
 constexpr int kMaxSplits = 16; // parts per key-split tile
 
 // Combines the parts of the key-split tiles: out[row] = sum_z O_z 2^(m_z - M) / sum_z l_z 2^(m_z - M),
@@ -1200,19 +1153,8 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnArgs a, int b
 }
 
 // Whole tiles first, then (tail.splits > 1) the tiles of the last round in parts, then the merge.
-// The role-split build (attn_pair.hpp) runs prepared bf16 operands on the 8-wave shape when the
-// measurement knob asks for it; it reads a quarter less from LDS per MFMA but takes 30 % more
-// cycles per key block than the single-role kernel, which stays the default.
-static bool g_role_split = false;
-
 template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
 static void launch_kernel(const AttnArgs& a, unsigned grid, hipStream_t stream) {
-    if constexpr (std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && QB == 1 && NW == 8) {
-        if (g_role_split) {
-            pairk::attn_pair_kernel<MASKED, BOUNDED><<<dim3(grid), dim3(512), pairk::kLdsAlloc, stream>>>(a);
-            return;
-        }
-    }
     attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
         <<<dim3(grid), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
 }
@@ -1329,8 +1271,7 @@ int attention_key_block() { return fwd::KB; }
 int attention_max_tokens() { return fwd::MAX_BLOCKS * fwd::KB; }
 
 hipError_t launch_attention(const AttnArgs& a, int in_dtype, int k_mode, int shape, hipStream_t stream) {
-    fwd::g_role_split = (shape & 2) != 0;
-    switch (shape & 1) {
+    switch (shape) {
     case 0: return fwd::launch_shape<1, 8>(a, in_dtype, k_mode, stream);
     case 1: return fwd::launch_shape<1, 4>(a, in_dtype, k_mode, stream);
     default: return hipErrorInvalidValue;
@@ -1339,11 +1280,6 @@ hipError_t launch_attention(const AttnArgs& a, int in_dtype, int k_mode, int sha
 
 hipError_t attention_setup() {
     hipError_t e;
-#define ZD_RAISE_PAIR(M, B) \
-    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd::pairk::attn_pair_kernel<M, B>), \
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)fwd::pairk::kLdsAlloc)) != hipSuccess) return e;
-    ZD_RAISE_PAIR(false, false) ZD_RAISE_PAIR(false, true) ZD_RAISE_PAIR(true, false) ZD_RAISE_PAIR(true, true)
-#undef ZD_RAISE_PAIR
     if ((e = fwd::raise_shape<1, 8>()) != hipSuccess) return e;
     if ((e = fwd::raise_shape<1, 4>()) != hipSuccess) return e;
     return hipSuccess;

@@ -103,6 +103,17 @@ struct PrepPair {
     int32_t pad0;
 };
 
+// Norm weights that the pre-pass cannot take as they lie (two element types, or off a
+// 16-byte boundary): 128 weights of Q and of K, each of its own type (kF32, kF16, kBF16)
+// at an element-aligned address, copied as f32 to out[0..127] and out[128..255].
+struct WeightStageArgs {
+    const void* q;
+    const void* k;
+    float* out;
+    int32_t q_dtype, k_dtype;
+};
+hipError_t launch_weight_stage(const WeightStageArgs& args, hipStream_t stream);
+
 // Kernel shape: 0 = 8 waves x 32 query rows (one workgroup per CU, 8-stage LDS
 // ring), 1 = 4 waves x 32 query rows (two workgroups per CU, 4-stage rings).
 int attention_block_rows(int shape);

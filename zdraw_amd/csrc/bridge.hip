@@ -52,15 +52,20 @@ struct Buffer {
     void* ptr;
     size_t len;
     bool owned;
+    // The bytes can only change through zdraw_hip_write_buffer: memory this library allocated,
+    // whose address was never handed out and which no kernel was ever asked to write. Only
+    // such buffers have anything read from them cached (the norm weights' maximum).
+    bool stable;
 };
-constexpr int kScratchSlots = 7;
+constexpr int kScratchSlots = 8; // per queue: slots 0-6 as below, 7 = staged norm weights
+constexpr int kCallerSlots = 7;  // zdraw_hip_attn_scratch hands these out (metal_api.m:6147-6191)
 struct Queue {
     Device* dev;
     hipStream_t stream;
     // The library's own scratch (prepared operands, parts of split tiles, rounded activations):
     // grow-only slots owned by the queue whose work uses them, so that two queues never share a
     // byte of it; freed with the queue.
-    Buffer* scratch[kScratchSlots] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    Buffer* scratch[kScratchSlots] = {};
 };
 struct Pipeline {
     int kind; // 0 = attention_block_mfma, 1 = qk_norm_rope, 2 = gemm_half
@@ -79,7 +84,7 @@ uint64_t g_dispatch = 0;
 uint64_t g_command = 0;
 uint64_t g_fallback = 0;
 uint64_t g_gpu_ns = 0;
-int g_variant = 0; // bit 0: kernel shape, 0 = 8 waves per workgroup, 1 = 4 waves (two workgroups per CU); bit 1: never split tail tiles; bit 2: the role-split build where it applies (prepared bf16 operands, 8-wave shape)
+int g_variant = 0; // bit 0: kernel shape, 0 = 8 waves per workgroup, 1 = 4 waves (two workgroups per CU); bit 1: never split tail tiles
 bool g_setup_done = false;
 bool g_gemm_setup_done = false;
 
@@ -205,7 +210,7 @@ Buffer* grow_slot(Buffer** slot_ptr, int slot, size_t bytes, Wait wait) {
         cur->len = bytes;
         return cur;
     }
-    *slot_ptr = new Buffer{p, bytes, true};
+    *slot_ptr = new Buffer{p, bytes, true, false};
     return *slot_ptr;
 }
 
@@ -241,7 +246,9 @@ struct FusedPlan {
     PrepArgs prep_v; // f32 operands only: V rounded to bf16 by the same launch
     bool round_v = false;
     int prep_in_dtype = kF32; // element type the pre-pass reads
-    int w_dtype = kF32; // element type of the norm weights (16-bit only with the pre-pass)
+    int w_dtype = kF32; // element type of the norm weights as the kernels read them (16-bit only with the pre-pass)
+    bool stage_w = false;  // the norm weights are first copied as f32 into scratch (two types, or off a 16-byte boundary)
+    WeightStageArgs stage;
 };
 
 // Norm weights as QkNormParams describes them (metal_c.zig:258-274): element
@@ -256,8 +263,9 @@ int norm_weight_dtype(uint32_t coded) {
 }
 
 // max |w| over the 128 norm weights at `off` in `b`, element type `dtype` (kF32, kF16, kBF16).
-// The weights live on the device: they are read back once per (address, type) and the figure is
-// kept until the buffer is written through this library or released. +inf if they cannot be
+// Only for buffers whose bytes cannot change behind the library's back (Buffer::stable): those
+// are read back once per (address, type) and the figure is kept until the buffer is written
+// through this library or released. +inf for any other buffer, and when the weights cannot be
 // read or hold a NaN (the caller then gets the running-maximum softmax).
 struct WeightMax {
     const void* ptr;
@@ -265,6 +273,16 @@ struct WeightMax {
     float amax;
 };
 std::vector<WeightMax> g_weight_max;
+
+// A buffer that a kernel is about to write, or whose address leaves the library: nothing read
+// from it is cached from here on.
+void forget_weight_max(const Buffer* b);
+void mark_unstable(void* handle) {
+    Buffer* b = static_cast<Buffer*>(handle);
+    if (!b || !b->stable) return;
+    b->stable = false;
+    if (b->ptr) forget_weight_max(b);
+}
 
 void forget_weight_max(const Buffer* b) {
     const char* lo = static_cast<const char*>(b->ptr);
@@ -281,6 +299,7 @@ void forget_weight_max(const Buffer* b) {
 }
 
 float weight_abs_max(const Buffer* b, uint64_t off, int dtype) {
+    if (!b->stable) return INFINITY;
     const void* src = static_cast<const char*>(b->ptr) + off;
     for (const WeightMax& w : g_weight_max)
         if (w.ptr == src && w.dtype == dtype) return w.amax;
@@ -374,6 +393,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     if ((why = check_operand(ok, x->in_dtype, x->batch, p->tokens, p->heads, "k"))) return invalid(why);
     if ((why = check_operand(ov, x->in_dtype, x->batch, p->tokens, p->heads, "v"))) return invalid(why);
     if ((why = check_operand(oo, x->out_dtype, x->batch, p->tokens, p->heads, "out"))) return invalid(why);
+    mark_unstable(out); // a kernel is about to write it
 
     AttnArgs a;
     memset(&a, 0, sizeof(a));
@@ -403,29 +423,47 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         if (!ops) return invalid("qk_mode set without operands");
         int qwd = kF32, kwd = kF32;
         uint64_t qwo = 0, kwo = 0;
+        bool stage = false;
         if (nw) {
             qwd = norm_weight_dtype(nw->q_dtype);
             kwd = norm_weight_dtype(nw->k_dtype);
             qwo = nw->q_off;
             kwo = nw->k_off;
-            if (qwd < 0 || kwd < 0 || qwd != kwd) return unavailable("norm weight dtype");
-            if (qwd != kF32 && x->k_site != ZDRAW_HIP_K_PREPASS) return unavailable("16-bit norm weights need the pre-pass");
-            if (qwo % 16 != 0 || kwo % 16 != 0) return invalid("norm weight offsets must be 16-byte aligned");
+            if (qwd < 0 || kwd < 0) return unavailable("norm weight dtype");
+            if (qwo % (qwd == kF32 ? 4 : 2) != 0 || kwo % (kwd == kF32 ? 4 : 2) != 0)
+                return invalid("norm weight offset is not a multiple of the element size");
             if (ops->q_weight_txt || ops->k_weight_txt) return invalid("text norm weights with typed norm weights");
         }
-        const size_t wbytes = (size_t)kHeadDim * (qwd == kF32 ? 4 : 2);
-        if (!ops->q_weight || !ops->k_weight || qwo > static_cast<Buffer*>(ops->q_weight)->len ||
-            kwo > static_cast<Buffer*>(ops->k_weight)->len ||
-            static_cast<Buffer*>(ops->q_weight)->len - qwo < wbytes || static_cast<Buffer*>(ops->k_weight)->len - kwo < wbytes ||
-            !static_cast<Buffer*>(ops->q_weight)->ptr || !static_cast<Buffer*>(ops->k_weight)->ptr)
+        const size_t qwbytes = (size_t)kHeadDim * (qwd == kF32 ? 4 : 2), kwbytes = (size_t)kHeadDim * (kwd == kF32 ? 4 : 2);
+        const Buffer* qwb = static_cast<Buffer*>(ops->q_weight);
+        const Buffer* kwb = static_cast<Buffer*>(ops->k_weight);
+        if (!qwb || !kwb || !qwb->ptr || !kwb->ptr || qwo > qwb->len || kwo > kwb->len || qwb->len - qwo < qwbytes ||
+            kwb->len - kwo < kwbytes)
             return invalid("norm weights must be [128] buffers (f32 unless the caller states a type)");
-        plan->w_dtype = qwd;
+        const bool q_al = ((uintptr_t)qwb->ptr + qwo) % 16 == 0, k_al = ((uintptr_t)kwb->ptr + kwo) % 16 == 0;
+        if (nw) {
+            // The kernels read the weights with 16-byte loads and one type for both operands
+            // (16-bit types only in the pre-pass). What a checkpoint view hands over instead (a
+            // type per operand, a file offset) is first copied as f32 into scratch.
+            stage = qwd != kwd || !q_al || !k_al || (qwd != kF32 && x->k_site != ZDRAW_HIP_K_PREPASS);
+        } else if (!q_al || !k_al) {
+            return invalid("norm weights must be 16-byte aligned");
+        }
+        plan->w_dtype = stage ? (int)kF32 : qwd;
         if ((ops->q_weight_txt && !need(ops->q_weight_txt, kHeadDim * 4)) ||
             (ops->k_weight_txt && !need(ops->k_weight_txt, kHeadDim * 4)))
             return invalid("text norm weights must be f32[128] buffers");
         if (!(x->eps >= 0.0f)) return invalid("eps");
-        a.q_w = reinterpret_cast<const float*>(static_cast<const char*>(static_cast<Buffer*>(ops->q_weight)->ptr) + qwo);
-        a.k_w = reinterpret_cast<const float*>(static_cast<const char*>(static_cast<Buffer*>(ops->k_weight)->ptr) + kwo);
+        a.q_w = reinterpret_cast<const float*>(static_cast<const char*>(qwb->ptr) + qwo);
+        a.k_w = reinterpret_cast<const float*>(static_cast<const char*>(kwb->ptr) + kwo);
+        if (stage) {
+            float* staged = static_cast<float*>(src->get(7, 2 * kHeadDim * sizeof(float)));
+            if (!staged) return scratch_failed(src);
+            plan->stage_w = true;
+            plan->stage = WeightStageArgs{a.q_w, a.k_w, staged, qwd, kwd};
+            a.q_w = staged;
+            a.k_w = staged + kHeadDim;
+        }
         a.q_w_txt = ops->q_weight_txt ? static_cast<const float*>(static_cast<Buffer*>(ops->q_weight_txt)->ptr) : nullptr;
         a.k_w_txt = ops->k_weight_txt ? static_cast<const float*>(static_cast<Buffer*>(ops->k_weight_txt)->ptr) : nullptr;
         a.qk.txt_rows = (int32_t)x->txt_rows;
@@ -435,9 +473,10 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
             // The caller asks for the form without a running maximum. Whether the scores allow it
             // is a function of the norm weights alone (rows normalised to sqrt(128) max|w|, a rope
             // that rotates): the library forms that bound itself, so a caller's figure that is too
-            // small cannot make the exponentials overflow.
-            float mq = weight_abs_max(static_cast<Buffer*>(ops->q_weight), qwo, qwd);
-            float mk = weight_abs_max(static_cast<Buffer*>(ops->k_weight), kwo, kwd);
+            // small cannot make the exponentials overflow. (Weight buffers that can change behind
+            // the library's back give +inf: the running-maximum form.)
+            float mq = weight_abs_max(qwb, qwo, qwd);
+            float mk = weight_abs_max(kwb, kwo, kwd);
             if (ops->q_weight_txt) mq = fmaxf(mq, weight_abs_max(static_cast<Buffer*>(ops->q_weight_txt), 0, kF32));
             if (ops->k_weight_txt) mk = fmaxf(mk, weight_abs_max(static_cast<Buffer*>(ops->k_weight_txt), 0, kF32));
             const float own = sqrtf((float)kHeadDim) * mq * mk * 1.02f; // 2 % for the roundings of norm and operands
@@ -629,6 +668,14 @@ int enqueue(const FusedPlan& plan, hipStream_t stream, bool no_alloc = false) {
         }
         g_setup_done = true;
     }
+    if (plan.stage_w) {
+        hipError_t e = launch_weight_stage(plan.stage, stream);
+        if (e != hipSuccess) {
+            set_err("norm weight staging launch: %s", hipGetErrorString(e));
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        g_dispatch++;
+    }
     if (plan.prepass) {
         const PrepArgs ops[3] = {plan.prep_q, plan.prep, plan.prep_v};
         hipError_t e = launch_qk_prepass(ops, plan.round_v ? 3 : 2, plan.prep_in_dtype, stream);
@@ -652,7 +699,7 @@ int enqueue(const FusedPlan& plan, hipStream_t stream, bool no_alloc = false) {
     TracePair tp{nullptr, nullptr};
     if (g_trace && !no_alloc && hipEventCreate(&tp.a) == hipSuccess && hipEventCreate(&tp.b) == hipSuccess)
         (void)hipEventRecord(tp.a, stream);
-    hipError_t e = launch_attention(args, plan.in_dtype, plan.k_mode, (g_variant & 1) | ((g_variant & 4) ? 2 : 0), stream);
+    hipError_t e = launch_attention(args, plan.in_dtype, plan.k_mode, g_variant & 1, stream);
     if (e != hipSuccess) {
         set_err("attention launch: %s", hipGetErrorString(e));
         return ZDRAW_HIP_ERR_HANDLE;
@@ -722,6 +769,7 @@ int enqueue_wide(Queue* queue, void* q, void* k, void* v, void* out, const Zdraw
         if (off % 16 != 0 || ((uintptr_t)bs[i]->ptr % 16) != 0) return invalid("operand not 16-byte aligned");
         if (off > bs[i]->len || n * 4 > bs[i]->len - off) return invalid("buffer smaller than [tokens][512] f32");
     }
+    mark_unstable(out);
     Buffer* sc[3];
     for (int i = 0; i < 3; i++) {
         sc[i] = queue_scratch(queue, i, (size_t)n * 2);
@@ -794,10 +842,12 @@ int finish_blocking(Queue* qu, hipEvent_t start, hipEvent_t stop) {
     return ZDRAW_HIP_OK;
 }
 
-Buffer* g_scratch[kScratchSlots] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+Buffer* g_scratch[kCallerSlots] = {};
 
 void* ScratchSource::get(int slot, size_t bytes) {
-    if (dry) return reinterpret_cast<void*>(uintptr_t{256}); // never dereferenced: the plan is not launched
+    // a plan of which only the pre-pass arguments are used: its operand slots are never
+    // dereferenced, the staged norm weights (slot 7) are
+    if (dry && slot != 7) return reinterpret_cast<void*>(uintptr_t{256});
     if (span) {
         const size_t at = (used + 255) & ~size_t{255};
         if (bytes > cap || at > cap - bytes) {
@@ -860,6 +910,7 @@ int enqueue_gemm_group(void* a, void* const* ws, void* const* cs, const uint64_t
         if (w_offs[i] > wb->len || w_bytes > wb->len - w_offs[i]) return invalid("W buffer too small");
         if (x->c_off > cb->len || c_bytes > cb->len - x->c_off) return invalid("C buffer too small");
     }
+    for (int i = 0; i < groups; i++) mark_unstable(cs[i]); // kernels are about to write them
     if (!g_gemm_setup_done) {
         hipError_t e = gemm_setup();
         if (e != hipSuccess) {
@@ -949,9 +1000,6 @@ void* zdraw_hip_create_device(void) {
         return nullptr;
     }
     if (hipSetDevice(0) != hipSuccess) return nullptr;
-    // ZDRAW_ATTN_VARIANT picks the kernel build for a whole process (measurement aid)
-    if (const char* v = getenv("ZDRAW_ATTN_VARIANT")) zdraw_hip_set_attention_variant(atoi(v));
-    if (const char* v = getenv("ZDRAW_GEMM_BUILD")) gemm_set_build(atoi(v));
     // One-time setup with the device current: the attention kernels' LDS limits (this also loads
     // their code), and this device's address of the no-allocation entry's scratch array.
     if (!g_setup_done) {
@@ -983,25 +1031,35 @@ void* zdraw_hip_create_queue(void* device) {
     Device* d = static_cast<Device*>(device);
     if (!d) return nullptr;
     hipStream_t s;
-    // Measurement aid: ZDRAW_HIP_CU_COUNT = n confines the stream to n compute units (mask bit
-    // i set for i < n; the driver deals the bits out over the XCDs in turn). It answers "does
-    // the kernel's time depend on how many CUs it has, or on the board's power limit".
-    const char* cus = getenv("ZDRAW_HIP_CU_COUNT");
-    const int ncu = cus ? atoi(cus) : 0;
-    if (ncu > 0 && ncu < d->cus) {
-        std::vector<uint32_t> mask((size_t)(d->cus + 31) / 32, 0u);
-        for (int i = 0; i < ncu; i++) mask[(size_t)i >> 5] |= 1u << (i & 31);
-        if (hipExtStreamCreateWithCUMask(&s, (uint32_t)mask.size(), mask.data()) != hipSuccess) {
-            set_err("hipExtStreamCreateWithCUMask failed");
-            return nullptr;
-        }
-        { Queue* nq = new Queue; nq->dev = d; nq->stream = s; return nq; }
-    }
     if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) {
         set_err("hipStreamCreate failed");
         return nullptr;
     }
-    { Queue* nq = new Queue; nq->dev = d; nq->stream = s; return nq; }
+    Queue* nq = new Queue;
+    nq->dev = d;
+    nq->stream = s;
+    return nq;
+}
+
+// Measurement aid (include/zdraw_hip_measure.h): a queue whose stream is confined to `cu_count`
+// compute units (mask bit i set for i < cu_count; the driver deals the bits out over the XCDs
+// in turn). It answers "does the kernel's time depend on how many CUs it has, or on the
+// board's power limit".
+void* zdraw_hip_create_queue_on_cus(void* device, int cu_count) {
+    Device* d = static_cast<Device*>(device);
+    if (!d) return nullptr;
+    if (cu_count <= 0 || cu_count >= d->cus) return zdraw_hip_create_queue(device);
+    hipStream_t s;
+    std::vector<uint32_t> mask((size_t)(d->cus + 31) / 32, 0u);
+    for (int i = 0; i < cu_count; i++) mask[(size_t)i >> 5] |= 1u << (i & 31);
+    if (hipExtStreamCreateWithCUMask(&s, (uint32_t)mask.size(), mask.data()) != hipSuccess) {
+        set_err("hipExtStreamCreateWithCUMask failed");
+        return nullptr;
+    }
+    Queue* nq = new Queue;
+    nq->dev = d;
+    nq->stream = s;
+    return nq;
 }
 
 void zdraw_hip_release_queue(void* queue) {
@@ -1027,7 +1085,7 @@ void* zdraw_hip_create_buffer(void* device, size_t size) {
         set_err("hipMalloc(%zu) failed", size);
         return nullptr;
     }
-    return new Buffer{p, size, true};
+    return new Buffer{p, size, true, true};
 }
 
 void* zdraw_hip_create_buffer_with_data(void* device, const uint8_t* data, size_t size) {
@@ -1042,9 +1100,41 @@ void* zdraw_hip_create_buffer_with_data(void* device, const uint8_t* data, size_
     return b;
 }
 
-void* zdraw_hip_create_buffer_no_copy(void* device, void* device_ptr, size_t size) {
-    if (!device || !device_ptr || size == 0) return nullptr;
-    return new Buffer{device_ptr, size, false};
+// metal_api.m:601-638 wraps the caller's host pages (unified memory). A discrete GPU reads its
+// own memory: the bytes are uploaded once and the caller keeps owning the source.
+void* zdraw_hip_create_buffer_no_copy(void* device, const uint8_t* data, size_t size) {
+    return zdraw_hip_create_buffer_with_data(device, data, size);
+}
+
+void* zdraw_hip_wrap_device_memory(void* device, void* device_ptr, size_t size) {
+    Device* d = static_cast<Device*>(device);
+    if (!d || !device_ptr || size == 0) return nullptr;
+    // only memory the runtime knows as a device allocation on this device, and only a range
+    // that lies inside that allocation, may reach a kernel
+    hipPointerAttribute_t attr;
+    memset(&attr, 0, sizeof(attr));
+    if (hipPointerGetAttributes(&attr, device_ptr) != hipSuccess) {
+        (void)hipGetLastError(); // a plain host pointer is reported as an error: clear it
+        set_err("wrap_device_memory: not memory the HIP runtime knows");
+        return nullptr;
+    }
+    if (attr.type != hipMemoryTypeDevice || attr.device != d->ordinal) {
+        set_err("wrap_device_memory: not device memory of device %d", d->ordinal);
+        return nullptr;
+    }
+    hipDeviceptr_t base = nullptr;
+    size_t span = 0;
+    if (hipMemGetAddressRange(&base, &span, device_ptr) != hipSuccess) {
+        (void)hipGetLastError();
+        set_err("wrap_device_memory: no allocation around the pointer");
+        return nullptr;
+    }
+    const uintptr_t lo = (uintptr_t)base, p = (uintptr_t)device_ptr;
+    if (p < lo || size > span || p - lo > span - size) {
+        set_err("wrap_device_memory: %zu bytes do not fit the allocation", size);
+        return nullptr;
+    }
+    return new Buffer{device_ptr, size, false, false};
 }
 
 void zdraw_hip_read_buffer(void* buffer, uint8_t* dst, size_t size) {
@@ -1067,7 +1157,18 @@ size_t zdraw_hip_buffer_length(void* buffer) {
 
 void* zdraw_hip_buffer_device_ptr(void* buffer) {
     Buffer* b = static_cast<Buffer*>(buffer);
-    return b ? b->ptr : nullptr;
+    if (!b) return nullptr;
+    mark_unstable(b); // whoever holds the address can write the bytes
+    return b->ptr;
+}
+
+int zdraw_hip_read_buffer_any(void* queue, void* buffer, uint8_t* dst, size_t size) {
+    Queue* q = static_cast<Queue*>(queue);
+    Buffer* b = static_cast<Buffer*>(buffer);
+    if (!q || !b || !b->ptr || !dst || size > b->len) return ZDRAW_HIP_ERR_HANDLE;
+    hipError_t e = hipStreamSynchronize(q->stream);
+    if (e == hipSuccess) e = hipMemcpy(dst, b->ptr, size, hipMemcpyDeviceToHost);
+    return e == hipSuccess ? ZDRAW_HIP_OK : hip_fail(e, "read_buffer_any");
 }
 
 void zdraw_hip_release_buffer(void* buffer) {
@@ -1077,6 +1178,8 @@ void zdraw_hip_release_buffer(void* buffer) {
     if (b->owned && b->ptr) (void)hipFree(b->ptr);
     delete b;
 }
+
+void zdraw_hip_release_weight_buffer(void* buffer) { zdraw_hip_release_buffer(buffer); }
 
 // ---------------------------------------------------------------- pipelines
 void* zdraw_hip_compile(void* device, const char* source, const char* entry, char* error_buf, size_t error_len) {
@@ -1266,6 +1369,8 @@ int run_qk_norm_rope_impl(void* queue, void* pipeline, void* q, void* k, const Z
     // except the pre-pass arguments assembled below. Both operands are checked
     // before the first launch, so a refused call leaves q untouched.
     PrepArgs prs[2];
+    bool stage_w = false;
+    WeightStageArgs stage;
     for (int which = 0; which < 2; which++) {
         ZdrawAttnParams sp = *p;
         sp.heads = sp.kv_heads = which == 0 ? p->heads : p->kv_heads;
@@ -1293,6 +1398,17 @@ int run_qk_norm_rope_impl(void* queue, void* pipeline, void* q, void* k, const Z
         pr.out_dtype = kF32;
         pr.scale = 1.0f;
         prs[which] = pr;
+        // both plans stage the same two weight vectors into the same place: one launch serves both
+        stage_w = plan.stage_w;
+        stage = plan.stage;
+    }
+    if (stage_w) {
+        hipError_t e = launch_weight_stage(stage, qu->stream);
+        if (e != hipSuccess) {
+            set_err("norm weight staging launch: %s", hipGetErrorString(e));
+            return ZDRAW_HIP_ERR_HANDLE;
+        }
+        g_dispatch++;
     }
     for (int which = 0; which < 2; which++) {
         hipError_t e = launch_qk_prepass(&prs[which], 1, kF32, qu->stream);
@@ -1562,7 +1678,7 @@ int zdraw_hip_run_chain_attn_enc(void* batch, const ZdrawHipChainAttnBuffers* bu
 
 // ------------------------------------------------------------------ scratch
 void* zdraw_hip_attn_scratch(void* device, int slot, size_t bytes) {
-    if (!device || slot < 0 || slot >= kScratchSlots || bytes == 0) return nullptr;
+    if (!device || slot < 0 || slot >= kCallerSlots || bytes == 0) return nullptr;
     // The caller's slots (the reference's process-static set, metal_api.m:6147-6191). The
     // library's own scratch lives with its queues, so nothing of the library reads these.
     return grow_slot(&g_scratch[slot], slot, bytes, [] { (void)hipDeviceSynchronize(); });
@@ -1649,7 +1765,7 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
     return m;
 }
 
-void zdraw_hip_set_attention_variant(int variant) { g_variant = variant & 7; }
+void zdraw_hip_set_attention_variant(int variant) { g_variant = variant & 3; }
 
 void zdraw_hip_set_gemm_build(int build) { gemm_set_build(build); }
 

@@ -139,6 +139,32 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
     }
 }
 
+// Norm weights as a checkpoint view hands them over (metal/mqk.zig:77-102: a type per
+// operand, a file offset that is only element-aligned), copied one element per thread to
+// f32 where the pre-pass reads them with 16-byte loads.
+__global__ void __launch_bounds__(2 * D) norm_weight_stage_kernel(const WeightStageArgs a) {
+    const int i = (int)threadIdx.x & (D - 1);
+    const bool is_k = (int)threadIdx.x >= D;
+    const void* src = is_k ? a.k : a.q;
+    const int dt = is_k ? a.k_dtype : a.q_dtype;
+    float v;
+    if (dt == kF32) {
+        v = static_cast<const float*>(src)[i];
+    } else {
+        const unsigned short h = static_cast<const unsigned short*>(src)[i];
+        v = dt == kBF16 ? __uint_as_float((unsigned)h << 16) : (float)__builtin_bit_cast(_Float16, h);
+    }
+    a.out[threadIdx.x] = v;
+}
+
+hipError_t launch_weight_stage(const WeightStageArgs& a, hipStream_t stream) {
+    if (!a.q || !a.k || !a.out) return hipErrorInvalidValue;
+    for (int dt : {a.q_dtype, a.k_dtype})
+        if (dt != kF32 && dt != kF16 && dt != kBF16) return hipErrorInvalidValue;
+    norm_weight_stage_kernel<<<dim3(1), dim3(2 * D), 0, stream>>>(a);
+    return hipGetLastError();
+}
+
 // One launch covers `count` operands (1 to 3) of equal tokens/heads/batch: the first two are
 // normalised and rotated (same mode), a third is only rounded and re-laid (mode kQkNone).
 hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipStream_t stream) {

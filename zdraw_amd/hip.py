@@ -95,6 +95,9 @@ SYMBOLS = {
     "zdraw_hip_create_buffer": (_vp, [_vp, _sz]),
     "zdraw_hip_create_buffer_with_data": (_vp, [_vp, _vp, _sz]),
     "zdraw_hip_create_buffer_no_copy": (_vp, [_vp, _vp, _sz]),
+    "zdraw_hip_wrap_device_memory": (_vp, [_vp, _vp, _sz]),
+    "zdraw_hip_read_buffer_any": (_int, [_vp, _vp, _vp, _sz]),
+    "zdraw_hip_release_weight_buffer": (None, [_vp]),
     "zdraw_hip_read_buffer": (None, [_vp, _vp, _sz]),
     "zdraw_hip_write_buffer": (None, [_vp, _vp, _sz]),
     "zdraw_hip_buffer_length": (_sz, [_vp]),
@@ -142,6 +145,7 @@ SYMBOLS = {
     "zdraw_hip_queue_sync": (_int, [_vp]),
     "zdraw_hip_set_attention_variant": (None, [_int]),
     "zdraw_hip_set_gemm_build": (None, [_int]),
+    "zdraw_hip_create_queue_on_cus": (_vp, [_vp, _int]),
     "zdraw_hip_attention_tail_plan": (None, [_u64, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "zdraw_hip_gemm_tail_plan": (None, [_u32, _u32, _u32, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "zdraw_hip_zimage_axis_lens": (_int, [_u64, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
