@@ -117,12 +117,12 @@ def spin_up(L, ctx, res, ms):
     return n
 
 
-def side_leg(L, ctx, w, *, bounded=True, spin_ms=300.0, warm=10, steps=100):
+def side_leg(L, ctx, w, *, bounded=True, staging=0, spin_ms=300.0, warm=10, steps=100):
     """A short measurement of one workload outside the driver-timed region: whole step
     (pre-pass + attention, wall clock) and the attention kernel alone (its own HIP events)."""
     from zdraw_amd import hip, workloads as wl
 
-    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_PREPASS, bounded=bounded)
+    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_PREPASS, bounded=bounded, staging=staging)
     spin_up(L, ctx, res, spin_ms)
     timed_region(L, ctx, res, warm)
     wall, kern_ms = timed_region(L, ctx, res, steps)
@@ -486,6 +486,8 @@ def main():
                     help="where K's norm+rope runs: inside the K-block load, or one pre-pass kernel per call")
     ap.add_argument("--variant", type=int, default=0, help="kernel shape: 0 = 8 waves, 1 = 4 waves x 2 workgroups")
     ap.add_argument("--dynamic-max", action="store_true", help="withhold the score bound (running-maximum softmax)")
+    ap.add_argument("--staging", choices=["bf16", "f16"], default="bf16",
+                    help="element type of the prepared Q and K (the scores' MFMA operands); P and V are bf16 either way")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-side-legs", action="store_true",
                     help="skip the short untimed-by-value legs (other softmax form, other benchmark shapes, the GEMM, chain and wide-head paths)")
@@ -515,7 +517,8 @@ def main():
     L.zdraw_hip_set_attention_variant(args.variant)
     w = wl.by_name(args.workload, seed=0)
     k_site = hip.K_PREPASS if args.k_site == "prepass" else hip.K_IN_TILE_LOAD
-    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=k_site, bounded=not args.dynamic_max)
+    staging = hip.F16 if args.staging == "f16" else 0
+    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=k_site, bounded=not args.dynamic_max, staging=staging)
 
     # untimed: leave the idle power state, then the warm-up steps
     spun = spin_up(L, ctx, res, args.spinup_ms)
@@ -550,6 +553,7 @@ def main():
     # the other K site, for the record (short, untimed by the driver's clock)
     other = "tile" if args.k_site == "prepass" else "prepass"
     res.ext.k_site = hip.K_IN_TILE_LOAD if other == "tile" else hip.K_PREPASS
+    res.ext.staging = 0  # (the tile-load site stages bf16 only)
     timed_region(L, ctx, res, 20)
     o_wall, _ = timed_region(L, ctx, res, 100)
 
@@ -558,8 +562,9 @@ def main():
     # the same workload (no score bound from the caller), and the other benchmark shapes.
     side = {}
     if not args.no_side_legs:
-        dyn = side_leg(L, ctx, w, bounded=args.dynamic_max)  # the softmax form the timed region did not run
+        dyn = side_leg(L, ctx, w, bounded=args.dynamic_max, staging=staging)  # the softmax form the timed region did not run
         side["dyn"] = dyn
+        side["stg"] = side_leg(L, ctx, w, bounded=not args.dynamic_max, staging=0 if staging else hip.F16)  # the other staging type
         for name in ("klein_512_x4", "zimage_1024", "klein_edit_ragged"):
             if name == w.name:
                 continue
@@ -598,13 +603,16 @@ def main():
             "k_norm_rope_site": args.k_site,
             "softmax": "running maximum" if args.dynamic_max else "bounded scores (QK-norm bound supplied by the caller)",
             "kernel_variant": args.variant,
+            "qk_staging": args.staging,
             "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
             f"tflops_with_k_site_{other}": flops / (o_wall / 100) / 1e12,
             "untimed_spinup_launches": spun,
             **({"cu_count": args.cu_count} if args.cu_count > 0 else {}),
             **({("tflops_bounded" if args.dynamic_max else "tflops_running_max"): side["dyn"]["value"],
                 ("kernel_frac_bounded" if args.dynamic_max else "kernel_frac_running_max"): side["dyn"]["kernel_frac"],
-                "other_workloads": {k: v for k, v in side.items() if k != "dyn"}} if side else {}),
+                ("tflops_bf16_staging" if staging else "tflops_f16_staging"): side["stg"]["value"],
+                ("kernel_frac_bf16_staging" if staging else "kernel_frac_f16_staging"): side["stg"]["kernel_frac"],
+                "other_workloads": {k: v for k, v in side.items() if k not in ("dyn", "stg")}} if side else {}),
         },
         "roofline": {
             "bound": "mfma",

@@ -90,7 +90,7 @@ typedef struct ZdrawHipAttnExt {
     uint64_t zimage_base[3];   /* Z-Image axis bases in pairs (zrope.Cache.axisBases) */
     uint32_t zimage_dims[3];   /* Z-Image axis widths, sum = head_dim */
     uint32_t batch;            /* independent segments, >= 1 */
-    uint32_t in_dtype;         /* ZDRAW_HIP_F32 or ZDRAW_HIP_BF16 */
+    uint32_t in_dtype;         /* ZDRAW_HIP_F32, ZDRAW_HIP_F16 or ZDRAW_HIP_BF16 (F16: with the pre-pass, or qk_mode NONE) */
     uint32_t out_dtype;        /* ZDRAW_HIP_F32, ZDRAW_HIP_F16 or ZDRAW_HIP_BF16 */
     uint32_t qk_mode;          /* ZDRAW_HIP_QK_* */
     uint32_t k_site;           /* ZDRAW_HIP_K_IN_TILE_LOAD or ZDRAW_HIP_K_PREPASS */
@@ -118,7 +118,14 @@ typedef struct ZdrawHipAttnExt {
      * (ZDRAW_HIP_F16 staging, see `staging`); scores reach sqrt(head_dim) * max|w_q| *
      * max|w_k| = 11.3 nats with unit weights and grow with the product of the weights. */
     float score_bound;
-    uint32_t reserved;
+    /* Element type in which the prepared Q and K are staged for the score product: 0 (or
+     * ZDRAW_HIP_BF16) = bf16, ZDRAW_HIP_F16 = IEEE half, the staging type of the reference's
+     * own kernels (klein/zflux2_glue_shader.zig:95-122, metal_api.m:6124-6145), values past
+     * +-65504 saturating as there: three more mantissa bits on every score at the same MFMA
+     * rate. It applies where the library writes the staged copies (qk_mode != NONE with
+     * k_site PREPASS, or f32 / f16 operands with qk_mode NONE); elsewhere F16 returns 1.
+     * in_dtype F16 implies it. P and V are bf16 in either case. */
+    uint32_t staging;
 } ZdrawHipAttnExt;
 
 /* Buffer handles for the fused entry's side operands (NULL where unused). */

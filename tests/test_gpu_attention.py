@@ -231,6 +231,78 @@ def test_f32_operands_are_rounded_once_and_take_the_16_bit_kernel(ctx, name):
     refimpl.check_close(outs[0], refimpl.reference_rows(w), name)
 
 
+# ------------------------------------- IEEE-half staging of the prepared Q and K
+@pytest.mark.parametrize("name", ["klein_1024", "klein_512_x4", "zimage_1024", "klein_edit_ragged"])
+@pytest.mark.parametrize("in_dtype", [hip.BF16, hip.F32, hip.F16], ids=["bf16", "f32", "f16"])
+@pytest.mark.parametrize("bounded", [True, False])
+def test_small_configs_with_half_precision_staging(ctx, name, in_dtype, bounded):
+    # the reference's kernels stage Q and K as IEEE half (klein/zflux2_glue_shader.zig:95-122):
+    # the pre-pass writes f16 copies and the scores run on the f16 MFMA; operands of every type
+    say(f"small config {name}, f16 staging, in_dtype={in_dtype} bounded={bounded}")
+    w = wl.by_name(name, seed=6, small=True)
+    res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_PREPASS, bounded=bounded, staging=hip.F16, in_dtype=in_dtype)
+    got = res.run()
+    again = res.run()
+    res.release()
+    want = refimpl.reference_rows(w)
+    mx, mean = refimpl.check_close(got, want, name + " (f16 staging)")
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    if in_dtype == hip.BF16:
+        # the same call with bf16 staging: three fewer mantissa bits on every score
+        res = wl.Resident(ctx, w, dtype=hip.BF16, k_site=hip.K_PREPASS, bounded=bounded)
+        base = res.run()
+        res.release()
+        err16 = np.abs(base.astype(np.float64) - want).mean()
+        say(f"  mean abs error: f16 staging {mean:.3e}, bf16 staging {err16:.3e}")
+        assert mean <= err16 * 1.05
+
+
+def test_half_precision_operands_used_as_given_and_refusals(ctx):
+    # qk_mode NONE: f16 operands (and f32 ones when the caller asks for f16 staging) are staged by
+    # one rounding launch at any length: Q with the softmax scale and K as f16, V as bf16
+    L = hip.lib()
+    rng = np.random.default_rng(77)
+    tokens, heads = 300, 2
+    shape = (tokens, heads, 128)
+    q, k, v = (rng.standard_normal(shape, dtype=np.float32) for _ in range(3))
+    cfg = zo.Config(tokens, heads, heads, 128)
+    h = lambda a: a.astype(np.float16)
+    want16 = zo.attention_run(h(q).astype(np.float32), h(k).astype(np.float32), h(v).astype(np.float32), cfg)
+
+    def call(in_dtype, staging, arrays, qk_mode=hip.QK_NONE, k_site=hip.K_PREPASS):
+        bufs = [ctx.buffer(a) for a in arrays]
+        o = ctx.buffer(nbytes=q.size * 4)
+        p = hip.AttnParams(tokens, heads, heads, 128, 0, 0)
+        x = hip.AttnExt()
+        for s_ in (x.q_stride, x.k_stride, x.v_stride, x.out_stride):
+            s_[0], s_[1], s_[2] = 0, heads * 128, 128
+        x.batch, x.in_dtype, x.out_dtype, x.qk_mode, x.k_site, x.staging = 1, in_dtype, hip.F32, qk_mode, k_site, staging
+        d0 = L.zdraw_hip_dispatch_count()
+        rc = L.zdraw_hip_run_attention_fused(ctx.queue, bufs[0].handle, bufs[1].handle, bufs[2].handle, o.handle,
+                                             C.byref(p), C.byref(x), C.byref(hip.QkOperands()))
+        out = o.read(np.float32, shape) if rc == 0 else None
+        launched = L.zdraw_hip_dispatch_count() - d0
+        for b in bufs + [o]:
+            b.release()
+        return rc, out, launched
+
+    rc, got, _ = call(hip.F16, 0, [h(q), h(k), h(v)])
+    assert rc == 0, hip.last_error()
+    refimpl.check_close(got, want16, "f16 operands, plain")
+    rc, got32, _ = call(hip.F32, hip.F16, [q, k, v])
+    assert rc == 0, hip.last_error()
+    refimpl.check_close(got32, zo.attention_run(q, k, v, cfg), "f32 operands, f16 staging, plain")
+    # f32 operands that hold f16 values give the bits of the f16 call
+    rc, same, _ = call(hip.F32, hip.F16, [h(q).astype(np.float32), h(k).astype(np.float32), h(v).astype(np.float32)])
+    assert rc == 0 and np.array_equal(same.view(np.uint32), got.view(np.uint32))
+    # refused, nothing enqueued: bf16 operands used as given cannot gain from f16 staging; the
+    # tile-load site prepares K as bf16 only; an unknown staging code is malformed
+    b16 = [host.f32_to_bf16_bits(a) for a in (q, k, v)]
+    assert call(hip.BF16, hip.F16, b16)[::2] == (hip.UNAVAILABLE, 0)
+    assert call(hip.F16, 0, [h(q), h(k), h(v)], qk_mode=hip.QK_KLEIN, k_site=hip.K_IN_TILE_LOAD)[::2] == (hip.UNAVAILABLE, 0)
+    assert call(hip.F32, 7, [q, k, v])[::2] == (hip.INVALID, 0)
+
+
 # ------------------------------------- configs 2-5, full size, sampled rows
 FULL = [("klein_1024", 48), ("klein_512_x4", 40), ("zimage_1024", 40), ("klein_edit_ragged", 28)]
 
@@ -759,8 +831,19 @@ def test_running_maximum_with_a_key_padding_mask_and_planted_keys(ctx):
     assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
 
 
-@pytest.mark.parametrize("k_site", [hip.K_IN_TILE_LOAD, hip.K_PREPASS])
-def test_planted_keys_through_norm_and_rope_without_a_score_bound(ctx, k_site):
+def score_scaled_bar(score_nats):
+    """The bar of the 16-bit path against the fp32 oracle as a function of the largest score.
+    Q' and K' are rounded to bf16 before the product (unit roundoff 2^-9 on each), so a score
+    of s nats carries an absolute error that grows like s * 2^-8, and a probability moves by
+    that many nats. The stated bar (2e-2 max, 2e-3 mean) is the one for unit norm weights,
+    where scores reach sqrt(128) = 11.3 nats; beyond that it scales with the score."""
+    f = max(1.0, float(score_nats) / float(np.sqrt(128.0)))
+    return refimpl.MAX_ABS * f, refimpl.MEAN_ABS * f
+
+
+@pytest.mark.parametrize("k_site,staging", [(hip.K_IN_TILE_LOAD, 0), (hip.K_PREPASS, 0), (hip.K_PREPASS, hip.F16)],
+                         ids=["tile", "prepass", "prepass-f16"])
+def test_planted_keys_through_norm_and_rope_without_a_score_bound(ctx, k_site, staging):
     # the fused Klein entry with norm weights far from one: the normalised scores spread over
     # tens of nats, the caller gives no bound, and the builds that prepare K in the tile load
     # (they subtract the reference) and in the pre-pass (scores arrive relative to it) must agree
@@ -777,21 +860,32 @@ def test_planted_keys_through_norm_and_rope_without_a_score_bound(ctx, k_site):
     wb = [ctx.buffer(a) for a in (wq, wk)]
     cos, sin = ctx.buffer(w.rope_cos), ctx.buffer(w.rope_sin)
     ctx.joint_klein(bufs[0], bufs[1], bufs[2], o, tokens=w.tokens, heads=w.heads, norm_q=wb[0], norm_k=wb[1],
-                    rope_cos=cos, rope_sin=sin, k_site=k_site, score_bound=0.0)
+                    rope_cos=cos, rope_sin=sin, k_site=k_site, score_bound=0.0, staging=staging)
     got = host.bf16_bits_to_f32(o.read(np.uint16, w.q.shape))[0]
     rb = lambda a: host.bf16_bits_to_f32(host.f32_to_bf16_bits(a))
+    r16 = (lambda a: a.astype(np.float16).astype(np.float32)) if staging == hip.F16 else rb
     qn = zo.klein_apply_rope(zo.klein_rms_norm_heads(rb(w.q[0]), wq), w.rope_cos, w.rope_sin)
     kn = zo.klein_apply_rope(zo.klein_rms_norm_heads(rb(w.k[0]), wk), w.rope_cos, w.rope_sin)
     scores = np.einsum("thd,shd->hts", qn, kn) / np.sqrt(128.0)
     assert scores.max() - np.median(scores) > 30.0 and scores.std() > 5.0  # the case is about a wide spread of scores
-    # With scores tens of nats apart the softmax is sharp, and the bf16 rounding of the prepared
-    # operands (a relative 2^-9 on every element) alone moves a probability by several percent:
-    # the oracle therefore takes the operands as the kernel's MFMAs see them, Q' = bf16(q' c) with
-    # c = log2(e) / sqrt(128) riding on it, K' = bf16(k'), and the usual bar applies
+    cfg = zo.Config(w.tokens, w.heads, w.heads, 128)
+    # (1) Against the oracle on the operands as the kernel's MFMAs see them, Q' = r16(q' c) with
+    # c = log2(e) / sqrt(128) riding on it, K' = r16(k'): what is left is P, V and the output in
+    # bf16, and the usual bar applies whatever the scores' size.
     c = np.float32(1.4426950408889634 / np.sqrt(128.0))
-    want = zo.attention_run(rb(qn * c) / c, rb(kn), rb(w.v[0]), zo.Config(w.tokens, w.heads, w.heads, 128))
-    mx, mean = refimpl.check_close(got, want, "klein, wide scores, no bound")
-    say(f"  max abs {mx:.2e} mean abs {mean:.2e}")
+    want_ops = zo.attention_run(r16(qn * c) / c, r16(kn), rb(w.v[0]), cfg)
+    mx, mean = refimpl.check_close(got, want_ops, "klein, wide scores, no bound (operands as staged)")
+    say(f"  vs oracle on the staged operands: max abs {mx:.2e} mean abs {mean:.2e}")
+    # (2) Against the oracle on the fp32 operands. With scores tens of nats apart the softmax is
+    # sharp and the rounding of Q' and K' alone moves a probability by several percent: the bar
+    # scales with the largest score for bf16 staging; IEEE-half staging (three more mantissa
+    # bits on both operands) is held to the unit-weight bar as it stands.
+    want = zo.attention_run(qn, kn, rb(w.v[0]), cfg)
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    bar_max, bar_mean = (refimpl.MAX_ABS, refimpl.MEAN_ABS) if staging == hip.F16 else score_scaled_bar(scores.max())
+    say(f"  vs the fp32 oracle: max abs {err.max():.2e} (bar {bar_max:.2e}) mean abs {err.mean():.2e} (bar {bar_mean:.2e}), "
+        f"largest score {scores.max():.1f} nats")
+    assert err.max() <= bar_max and err.mean() <= bar_mean
     for b in bufs + wb + [o, cos, sin]:
         b.release()
 

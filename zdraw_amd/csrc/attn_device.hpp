@@ -10,6 +10,8 @@
 namespace zdraw {
 
 typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -25,6 +27,7 @@ constexpr int D = kHeadDim;
 template <typename T> struct Raw8;
 template <> struct Raw8<float> { f32x4 a, b; };
 template <> struct Raw8<bf16_t> { u32x4 r; };
+template <> struct Raw8<f16_t> { u32x4 r; };
 
 template <typename T>
 __device__ __forceinline__ Raw8<T> ld_raw8(const T* p, bool ok) {
@@ -110,6 +113,11 @@ __device__ __forceinline__ void unpack8(const Raw8<bf16_t>& r, float (&x)[8]) {
         x[2 * i + 1] = __uint_as_float(r.r[i] & 0xffff0000u);
     }
 }
+__device__ __forceinline__ void unpack8(const Raw8<f16_t>& r, float (&x)[8]) {
+    const f16x8 h = __builtin_bit_cast(f16x8, r.r);
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[i] = (float)h[i];
+}
 
 // fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ u32x4 pack_bf16x8(const float (&x)[8]) {
@@ -118,6 +126,14 @@ __device__ __forceinline__ u32x4 pack_bf16x8(const float (&x)[8]) {
     for (int i = 0; i < 8; i++) v[i] = x[i];
     bf16x8 b = __builtin_convertvector(v, bf16x8);
     return __builtin_bit_cast(u32x4, b);
+}
+// fp32 -> IEEE half, round to nearest even. Values past the half range saturate at +-65504,
+// as the reference's staging kernels clamp them (metal_api.m:6138).
+__device__ __forceinline__ u32x4 pack_f16x8(const float (&x)[8]) {
+    f16x8 h;
+#pragma unroll
+    for (int i = 0; i < 8; i++) h[i] = (f16_t)fminf(fmaxf(x[i], -65504.0f), 65504.0f);
+    return __builtin_bit_cast(u32x4, h);
 }
 __device__ __forceinline__ u32x4 raw_to_bf16(const Raw8<bf16_t>& r) { return r.r; }
 __device__ __forceinline__ u32x4 raw_to_bf16(const Raw8<float>& r) {

@@ -101,7 +101,13 @@ __device__ __forceinline__ void pin(T& v) {
 // lazy running maximum is kept: S accumulates on top of minus the reference point
 // (the MFMA's C operand), so the exponentials need no subtraction either, and the
 // block's row sums, not a maximum per block, say when the reference must move.
-template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
+//
+// SF16: the prepared Q and K are IEEE half instead of bf16 (the staging type of the reference's
+// own kernels, klein/zflux2_glue_shader.zig:95-122) and S = K Q^T runs on
+// v_mfma_f32_32x32x16_f16: three more mantissa bits on every score at the same MFMA rate. P and
+// V stay bf16 (P reaches 2^64 in the bounded form). Only for the direct-to-LDS build, where the
+// operands' bits go from memory to the MFMA untouched.
+template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW, bool SF16 = false>
 __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(const AttnArgs a) {
     constexpr int NT = NW * 64;
     constexpr int QR = 32 * QB;       // query rows per wave
@@ -116,6 +122,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // conflicts are avoided by swizzling the 16-byte chunk position instead:
     // K chunk c of row r sits at c ^ (r & 15), V chunk c of row r at c ^ ((r & 3) << 2).
     constexpr bool DMA = kDirectLds && std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && NW == 8 && QB == 1;
+    static_assert(!SF16 || DMA, "half-precision score operands exist for the direct-to-LDS build only");
     // The product O^T += V^T P^T on v_mfma_f32_16x16x32 (the scores keep the 32 x 32 x 16 form, in
     // which a lane owns one query). The 16 x 16 form moves half the accumulator bytes per FLOP
     // through the register file, and at the board's power limit that is worth clock: -2 % of the
@@ -493,6 +500,14 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             (lds_s16x4_t)(vfo16[dt >> 1][dt & 1] + (unsigned)(stage * (VSTAGE * 2) + (8 * half) * (VROW * 2))));
     };
 
+    // one 32 x 32 x 16 step of S^T += K Q^T on the operands' element type
+    auto score_mfma = [&](const bf16x8& kfrag, const bf16x8& qfrag, const f32x16& c) __attribute__((always_inline)) -> f32x16 {
+        if constexpr (SF16)
+            return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kfrag), __builtin_bit_cast(f16x8, qfrag), c, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag, qfrag, c, 0, 0, 0);
+    };
+
     // S^T block = K(block) . Q^T for both query blocks
     auto qk_block = [&](int stage, f32x16 (&s_out)[QB]) {
 #pragma unroll
@@ -504,7 +519,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             const bf16x8 kf = k_frag(stage, s);
 #pragma unroll
             for (int qi = 0; qi < QB; qi++)
-                s_out[qi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qi][s], s_out[qi], 0, 0, 0);
+                s_out[qi] = score_mfma(kf, qf[qi][s], s_out[qi]);
         }
     };
 
@@ -619,7 +634,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
                 const int st = slot >> 1;
 #pragma unroll
                 for (int qi = 0; qi < QB; qi++)
-                    s_next[qi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st], qf[qi][st], s_next[qi], 0, 0, 0);
+                    s_next[qi] = score_mfma(kf[st], qf[qi][st], s_next[qi]);
             }
             if (MFMA_PRIO) __builtin_amdgcn_s_setprio(0);
         };
@@ -1155,6 +1170,13 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnArgs a, int b
 // Whole tiles first, then (tail.splits > 1) the tiles of the last round in parts, then the merge.
 template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
 static void launch_kernel(const AttnArgs& a, unsigned grid, hipStream_t stream) {
+    if constexpr (std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && QB == 1 && NW == 8) {
+        if (a.score_f16) {
+            attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW, true>
+                <<<dim3(grid), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
+            return;
+        }
+    }
     attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>
         <<<dim3(grid), dim3(NW * 64), lds_bytes(ring_stages(QB, NW)), stream>>>(a);
 }
@@ -1205,6 +1227,9 @@ template <typename TIn, int QB, int NW>
 static hipError_t launch_flags(const AttnArgs& a, int k_mode, hipStream_t stream) {
     // Q and K are prepared at the same site: the builds rely on it
     if ((k_mode == kQkNone) != (a.q_mode == kQkNone)) return hipErrorInvalidValue;
+    // half-precision score operands: prepared 16-bit rows on the eight-wave shape, scale already applied
+    if (a.score_f16 && !(std::is_same<TIn, bf16_t>::value && k_mode == kQkNone && QB == 1 && NW == 8 && a.scale_log2 == 1.0f))
+        return hipErrorInvalidValue;
     // the masked build is only needed when some key of some block is excluded
     const bool masked = a.key_pad != nullptr || (a.key_limit % KB) != 0;
     const bool bounded = a.bounded != 0;
@@ -1224,6 +1249,11 @@ static hipError_t launch_shape(const AttnArgs& a, int in_dtype, int k_mode, hipS
 
 template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
 static hipError_t raise_lds() {
+    if constexpr (std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && QB == 1 && NW == 8) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(ring_stages(QB, NW)));
+        if (e != hipSuccess) return e;
+    }
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(ring_stages(QB, NW)));
 }

@@ -56,7 +56,7 @@ struct AttnArgs {
     int32_t out_dtype;  // kF32, kF16 or kBF16
     float scale_log2;   // log2(e) / sqrt(head_dim)
     int32_t bounded;    // 1: scaled scores are known to fit the fp32 exponent with room to spare
-    int32_t pad1;
+    int32_t score_f16;  // 1: q and k hold IEEE half (prepared operands only): S = K Q^T runs on the f16 MFMA; v stays bf16
     QkOps qk;
     // QK-norm weights (f32[128]); *_txt used for tokens < qk.txt_rows when non-null
     const float* q_w;
@@ -88,7 +88,7 @@ struct PrepArgs {
     int64_t y_bs, y_ts, y_hs;
     int32_t tokens, heads, batch;
     int32_t mode;       // QkMode; kQkNone = the rows are only rounded and re-laid (V beside a prepared Q and K)
-    int32_t out_dtype;  // kF32 or kBF16
+    int32_t out_dtype;  // kF32, kF16 or kBF16 (per operand: a launch may write Q and K as f16 and V as bf16)
     float scale;        // multiplies the result (1 for K; log2(e)/sqrt(head_dim) when Q is prepared for attention)
     QkOps qk;
     const void* w;      // 128 norm weights, element type w_dtype

@@ -379,10 +379,21 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
     if (x->batch == 0) return invalid("batch == 0");
     const uint64_t max_tokens = (uint64_t)attention_max_tokens();
     if ((uint64_t)p->tokens > max_tokens) return unavailable("too many tokens");
-    if ((x->in_dtype != ZDRAW_HIP_F32 && x->in_dtype != ZDRAW_HIP_BF16) ||
+    if ((x->in_dtype != ZDRAW_HIP_F32 && x->in_dtype != ZDRAW_HIP_BF16 && x->in_dtype != ZDRAW_HIP_F16) ||
         (x->out_dtype != ZDRAW_HIP_F32 && x->out_dtype != ZDRAW_HIP_BF16 && x->out_dtype != ZDRAW_HIP_F16))
         return unavailable("activation dtype");
     if (x->qk_mode > ZDRAW_HIP_QK_ZIMAGE) return invalid("qk_mode");
+    if (x->staging != 0 && x->staging != ZDRAW_HIP_BF16 && x->staging != ZDRAW_HIP_F16) return invalid("staging");
+    // IEEE-half score operands (the reference's staging type): where the library writes the
+    // staged copies of Q and K itself, on the eight-wave kernel shape
+    const bool stage_f16 = x->in_dtype == ZDRAW_HIP_F16 || x->staging == ZDRAW_HIP_F16;
+    if (stage_f16) {
+        if (x->qk_mode != ZDRAW_HIP_QK_NONE && x->k_site != ZDRAW_HIP_K_PREPASS)
+            return unavailable("IEEE-half staging needs the pre-pass (k_site)");
+        if (x->qk_mode == ZDRAW_HIP_QK_NONE && x->in_dtype == ZDRAW_HIP_BF16)
+            return unavailable("IEEE-half staging of operands that arrive as bf16 and are used as given");
+        if (g_variant & 1) return unavailable("IEEE-half staging on the four-wave kernel shape");
+    }
 
     const Operand oq{static_cast<Buffer*>(q), x->q_off, x->q_stride[0], x->q_stride[1], x->q_stride[2]};
     const Operand ok{static_cast<Buffer*>(k), x->k_off, x->k_stride[0], x->k_stride[1], x->k_stride[2]};
@@ -553,10 +564,10 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         // half-precision head-major copies the same way): the pre-pass rounds Q and K to bf16
         // and the same launch rounds V into slot 2, so the attention kernel runs its
         // direct-to-LDS build on 16-bit rows instead of rounding every block it loads.
-        const bool to_bf16 = x->in_dtype == ZDRAW_HIP_F32;
-        const uint32_t prep_out = to_bf16 ? (uint32_t)ZDRAW_HIP_BF16 : x->in_dtype;
-        const size_t es = elem_size(prep_out);
-        const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * es;
+        // f32 and f16 operands: V needs a bf16 copy as well
+        const bool to_bf16 = x->in_dtype != ZDRAW_HIP_BF16;
+        const uint32_t prep_out = stage_f16 ? (uint32_t)ZDRAW_HIP_F16 : (uint32_t)ZDRAW_HIP_BF16;
+        const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * 2;
         void* sq = src->get(0, bytes);
         void* sk = src->get(1, bytes);
         if (!sq || !sk) return scratch_failed(src);
@@ -593,12 +604,15 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         plan->args.q_bs = pr.y_bs; plan->args.q_ts = pr.y_ts; plan->args.q_hs = pr.y_hs;
         plan->args.q_mode = kQkNone;
         plan->args.scale_log2 = 1.0f;
+        plan->args.score_f16 = stage_f16 ? 1 : 0;
         plan->prep_in_dtype = (int)x->in_dtype;
+        plan->in_dtype = kBF16; // the kernel's 16-bit build (its score operands' type is args.score_f16)
         if (to_bf16) {
             void* sv = src->get(2, bytes);
             if (!sv) return scratch_failed(src);
             PrepArgs pv = pr;
             pv.mode = kQkNone;
+            pv.out_dtype = kBF16;
             pv.x = a.v;
             pv.y = sv;
             pv.x_bs = a.v_bs; pv.x_ts = a.v_ts; pv.x_hs = a.v_hs;
@@ -611,11 +625,14 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
             plan->in_dtype = kBF16;
         }
     }
-    if (x->qk_mode == ZDRAW_HIP_QK_NONE && x->in_dtype == ZDRAW_HIP_F32 && p->tokens >= kRoundPlainTokens) {
+    if (x->qk_mode == ZDRAW_HIP_QK_NONE &&
+        ((x->in_dtype == ZDRAW_HIP_F32 && p->tokens >= kRoundPlainTokens) || stage_f16)) {
         // Plain attention on f32 rows (the reference's base entry, metal_c.zig:286-299, takes
         // them): Q (with the softmax scale), K and V are rounded to bf16 once, head-major, into
         // slots 0-2 by one launch, and the kernel is the direct-to-LDS build, as for prepared
-        // operands. Short sequences stay on the build that rounds in its tile load.
+        // operands. Short sequences stay on the build that rounds in its tile load. IEEE-half
+        // staging (f16 operands, or asked for on f32 ones) takes this way at any length: Q with
+        // its scale and K become f16 copies, V a bf16 one.
         const size_t bytes = (size_t)x->batch * p->heads * p->tokens * kHeadDim * 2;
         void* sc[3];
         for (int i = 0; i < 3; i++) {
@@ -632,6 +649,7 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         pr.out_dtype = kBF16;
         pr.scale = 1.0f;
         PrepArgs pq = pr, pk = pr, pv = pr;
+        pq.out_dtype = pk.out_dtype = stage_f16 ? (int32_t)kF16 : (int32_t)kBF16;
         pq.x = a.q; pq.y = sc[0]; pq.x_bs = a.q_bs; pq.x_ts = a.q_ts; pq.x_hs = a.q_hs; pq.scale = a.scale_log2;
         pk.x = a.k; pk.y = sc[1]; pk.x_bs = a.k_bs; pk.x_ts = a.k_ts; pk.x_hs = a.k_hs;
         pv.x = a.v; pv.y = sc[2]; pv.x_bs = a.v_bs; pv.x_ts = a.v_ts; pv.x_hs = a.v_hs;
@@ -640,8 +658,9 @@ int plan_attention(Device* dev, void* q, void* k, void* v, void* out, const Zdra
         plan->prep_v = pv;
         plan->round_v = true;
         plan->prepass = true;
-        plan->prep_in_dtype = kF32;
+        plan->prep_in_dtype = (int)x->in_dtype;
         plan->in_dtype = kBF16;
+        plan->args.score_f16 = stage_f16 ? 1 : 0;
         plan->args.q = sc[0];
         plan->args.k = sc[1];
         plan->args.v = sc[2];

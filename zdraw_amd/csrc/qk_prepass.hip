@@ -59,7 +59,7 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
                     *reinterpret_cast<f32x4*>(dst) = f32x4{x[0], x[1], x[2], x[3]};
                     *reinterpret_cast<f32x4*>(dst + 4) = f32x4{x[4], x[5], x[6], x[7]};
                 } else {
-                    *reinterpret_cast<u32x4*>(reinterpret_cast<bf16_t*>(p.y) + off) = pack_bf16x8(x);
+                    *reinterpret_cast<u32x4*>(reinterpret_cast<bf16_t*>(p.y) + off) = p.out_dtype == kF16 ? pack_f16x8(x) : pack_bf16x8(x);
                 }
             }
         }
@@ -133,7 +133,7 @@ __global__ void __launch_bounds__(kPrepTokens * 64) qk_prepass_kernel(const Prep
                 *reinterpret_cast<f32x4*>(dst) = f32x4{x[0], x[1], x[2], x[3]};
                 *reinterpret_cast<f32x4*>(dst + 4) = f32x4{x[4], x[5], x[6], x[7]};
             } else {
-                *reinterpret_cast<u32x4*>(reinterpret_cast<bf16_t*>(p.y) + off) = pack_bf16x8(x);
+                *reinterpret_cast<u32x4*>(reinterpret_cast<bf16_t*>(p.y) + off) = p.out_dtype == kF16 ? pack_f16x8(x) : pack_bf16x8(x);
             }
         }
     }
@@ -199,6 +199,9 @@ hipError_t launch_qk_prepass(const PrepArgs* ops, int count, int in_dtype, hipSt
     } else if (in_dtype == kBF16) {
         if (klein) ZD_PREP(bf16_t, kQkKlein);
         else ZD_PREP(bf16_t, kQkZimage);
+    } else if (in_dtype == kF16) {
+        if (klein) ZD_PREP(f16_t, kQkKlein);
+        else ZD_PREP(f16_t, kQkZimage);
     } else {
         return hipErrorInvalidValue;
     }

@@ -33,7 +33,7 @@ class AttnExt(C.Structure):
         ("zimage_base", C.c_uint64 * 3), ("zimage_dims", C.c_uint32 * 3),
         ("batch", C.c_uint32), ("in_dtype", C.c_uint32), ("out_dtype", C.c_uint32),
         ("qk_mode", C.c_uint32), ("k_site", C.c_uint32), ("txt_rows", C.c_uint32), ("eps", C.c_float),
-        ("score_bound", C.c_float), ("reserved", C.c_uint32),
+        ("score_bound", C.c_float), ("staging", C.c_uint32),
     ]
 
 

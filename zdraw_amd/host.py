@@ -93,7 +93,7 @@ class _Klein(C.Structure):
                 ("norm_added_q", C.c_void_p), ("norm_added_k", C.c_void_p),
                 ("rope_cos", C.c_void_p), ("rope_sin", C.c_void_p), ("rope_per_segment", C.c_bool),
                 ("key_pad", C.c_void_p), ("out_row_stride", C.c_size_t), ("k_site", C.c_uint32),
-                ("score_bound", C.c_float)]
+                ("score_bound", C.c_float), ("staging", C.c_uint32)]
 
 
 class _Zimage(C.Structure):
@@ -102,7 +102,7 @@ class _Zimage(C.Structure):
                 ("tokens", C.c_size_t), ("heads", C.c_size_t),
                 ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("pos", C.c_void_p), ("rope_pairs", C.c_void_p),
                 ("dims", C.c_size_t * 3), ("bases", C.c_size_t * 3), ("norm_eps", C.c_float),
-                ("k_site", C.c_uint32), ("score_bound", C.c_float)]
+                ("k_site", C.c_uint32), ("score_bound", C.c_float), ("staging", C.c_uint32)]
 
 
 class _RopeCache(C.Structure):
@@ -290,19 +290,19 @@ class Context:
     def joint_klein(self, q, k, v, o, *, tokens, heads, nb=1, in_dtype=hip.BF16, out_dtype=hip.BF16,
                     norm_q, norm_k, norm_added_q=None, norm_added_k=None, txt_rows=0,
                     rope_cos, rope_sin, rope_per_segment=False, key_pad=None,
-                    out_row_stride=0, k_site=hip.K_IN_TILE_LOAD, score_bound=0.0):
+                    out_row_stride=0, k_site=hip.K_IN_TILE_LOAD, score_bound=0.0, staging=0):
         h = lambda b: b.handle if b is not None else None
         c = _Klein(h(q), h(k), h(v), h(o), in_dtype, out_dtype, tokens, heads, nb, txt_rows,
                    h(norm_q), h(norm_k), h(norm_added_q), h(norm_added_k), h(rope_cos), h(rope_sin),
-                   rope_per_segment, h(key_pad), out_row_stride, k_site, score_bound)
+                   rope_per_segment, h(key_pad), out_row_stride, k_site, score_bound, staging)
         _raise(lib().zh_joint_klein(self._ptr, C.byref(c)))
 
     def joint_zimage(self, q, k, v, o, *, tokens, heads, in_dtype=hip.BF16, out_dtype=hip.BF16,
                      q_norm, k_norm, pos, rope_pairs, dims, bases, norm_eps, k_site=hip.K_IN_TILE_LOAD,
-                     score_bound=0.0):
+                     score_bound=0.0, staging=0):
         c = _Zimage(q.handle, k.handle, v.handle, o.handle, in_dtype, out_dtype, tokens, heads,
                     q_norm.handle, k_norm.handle, pos.handle, rope_pairs.handle,
-                    (C.c_size_t * 3)(*dims), (C.c_size_t * 3)(*bases), norm_eps, k_site, score_bound)
+                    (C.c_size_t * 3)(*dims), (C.c_size_t * 3)(*bases), norm_eps, k_site, score_bound, staging)
         _raise(lib().zh_joint_zimage(self._ptr, C.byref(c)))
 
     def qk_run(self, q_buf, k_buf, q_weight, k_weight, pos, rope_values, dims, lens, *, tokens, heads,

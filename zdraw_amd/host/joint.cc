@@ -122,6 +122,7 @@ Error run(hattn::Context* ctx, const Klein& c) {
     x.rope_batch_rows = c.rope_per_segment ? c.tokens : 0;
     x.mask_batch_bytes = c.key_pad ? c.tokens : 0;
     x.score_bound = c.score_bound;
+    x.staging = c.staging;
     ZdrawHipQkOperands ops;
     memset(&ops, 0, sizeof(ops));
     ops.q_weight = c.norm_q;
@@ -157,6 +158,7 @@ Error run(hattn::Context* ctx, const Zimage& c) {
     x.k_site = (uint32_t)c.k_site;
     x.eps = c.norm_eps;
     x.score_bound = c.score_bound;
+    x.staging = c.staging;
     for (int a = 0; a < 3; a++) {
         x.zimage_dims[a] = (uint32_t)c.dims[a];
         x.zimage_base[a] = c.bases[a];

@@ -165,6 +165,7 @@ struct Klein {
     size_t out_row_stride;               // elements between output token rows; 0 = heads*128
     KSite k_site;
     float score_bound;                   // see scoreBound(); 0 = unknown (running-maximum softmax)
+    uint32_t staging;                    // 0 = bf16 copies of the prepared Q and K; ZDRAW_HIP_F16 = IEEE half (needs the pre-pass)
 };
 Error run(hattn::Context* ctx, const Klein& c);
 
@@ -190,6 +191,7 @@ struct Zimage {
     float norm_eps;
     KSite k_site;
     float score_bound;                   // see scoreBound(); 0 = unknown
+    uint32_t staging;                    // as Klein::staging
 };
 Error run(hattn::Context* ctx, const Zimage& c);
 

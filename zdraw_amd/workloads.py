@@ -143,9 +143,14 @@ class Resident:
     """A workload's operands uploaded once; `launch()` enqueues one pass of the
     hot path (inputs already in HBM), `run()` also waits and reads O back."""
 
-    def __init__(self, ctx: host.Context, w: Workload, dtype=hip.BF16, k_site=hip.K_IN_TILE_LOAD, bounded=True):
+    def __init__(self, ctx: host.Context, w: Workload, dtype=hip.BF16, k_site=hip.K_IN_TILE_LOAD, bounded=True,
+                 staging=0, in_dtype=None):
+        """dtype: element type of the output (and of the operands unless in_dtype says otherwise);
+        staging: hip.F16 stages the prepared Q and K as IEEE half (needs the pre-pass)."""
         self.ctx, self.w, self.dtype, self.k_site = ctx, w, dtype, k_site
-        conv = host.f32_to_bf16_bits if dtype == hip.BF16 else (lambda a: np.ascontiguousarray(a, np.float32))
+        in_dtype = dtype if in_dtype is None else in_dtype
+        conv = {hip.BF16: host.f32_to_bf16_bits, hip.F16: (lambda a: np.ascontiguousarray(a, np.float16)),
+                hip.F32: (lambda a: np.ascontiguousarray(a, np.float32))}[in_dtype]
         self.q = ctx.buffer(conv(w.q))
         self.k = ctx.buffer(conv(w.k))
         self.v = ctx.buffer(conv(w.v))
@@ -165,7 +170,7 @@ class Resident:
             s[0] = w.tokens * hidden if w.batch > 1 else 0
             s[1] = hidden
             s[2] = HEAD_DIM
-        x.batch, x.in_dtype, x.out_dtype, x.k_site = w.batch, dtype, dtype, k_site
+        x.batch, x.in_dtype, x.out_dtype, x.k_site, x.staging = w.batch, in_dtype, dtype, k_site, staging
         if w.kind == "plain":
             x.qk_mode = hip.QK_NONE
         elif w.kind == "klein":
