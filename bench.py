@@ -286,7 +286,7 @@ def chain_main(args):
     L = hip.lib()
     ctx = host.Context.init()
     w = wl.by_name("zimage_1024", seed=0)
-    tokens, heads = w.tokens, w.heads
+    tokens, heads = w.tokens, (args.chain_heads or w.heads)
     hidden = inner = heads * 128
     rng = np.random.default_rng(0)
     bits = lambda a: host.f32_to_bf16_bits(a)
@@ -353,10 +353,47 @@ def chain_main(args):
                      "unit": "TFLOP/s", "frac": flops / (dev_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
                      "kernel": "3 x gemm + qk_prepass + attn_fwd + gemm", "kernel_ms": dev_ms},
     }
+    if args.chain_check_rows and not act32:
+        line["parity_check"] = chain_check(w, tokens, heads, x, wall_w, out, args.chain_check_rows)
     for b in (nb, wb, qb, kb, vb, mixb, ob, ones, posb, ropeb):
         b.release()
     ctx.deinit()
     return line
+
+
+def chain_check(w, tokens, heads, x, weights, got, nrows):
+    """The segment's output rows `rows` against the oracle chain (runtime/ops.zig linear ->
+    zimage/zattn.zig norm -> rope -> attention.run -> linear) with the same bf16 hand-overs:
+    K and V of every token, Q and the output projection of the sampled rows only."""
+    import numpy as np
+
+    from oracle import zoracle as zo
+    from zdraw_amd import host
+    from zdraw_amd import workloads as wl
+
+    t0 = time.perf_counter()
+    rb = lambda a: host.bf16_bits_to_f32(host.f32_to_bf16_bits(np.ascontiguousarray(a, np.float32)))
+    rows = sorted(set(int(t) for t in np.random.default_rng(1).choice(tokens, nrows, replace=False)) | {0, tokens - 1})
+    xr, wr = rb(x), [rb(weights[i]) for i in range(4)]
+    cfg = zo.RopeConfig(wl.ZIMAGE_DIMS, wl.ZIMAGE_LENS, wl.ZIMAGE_THETA)
+    vals = zo.zrope_fill(cfg)
+    pos = np.ascontiguousarray(w.pos, dtype=np.uintp)
+    ones = np.ones(128, np.float32)
+    k = rb(zo.linear_batch(xr, wr[1])).reshape(tokens, heads, 128)
+    v = rb(zo.linear_batch(xr, wr[2])).reshape(tokens, heads, 128)
+    q = np.zeros((tokens, heads, 128), np.float32)
+    q[rows] = rb(zo.linear_batch(xr[rows], wr[0])).reshape(len(rows), heads, 128)
+    qn = np.zeros_like(q)
+    qn[rows] = zo.zimage_rotate(zo.zimage_norm_heads(q[rows], ones, wl.ZIMAGE_EPS), vals, cfg, pos[rows])
+    kn = zo.zimage_rotate(zo.zimage_norm_heads(k, ones, wl.ZIMAGE_EPS), vals, cfg, pos)
+    mix = zo.attention_token_list(qn, kn, v, zo.Config(tokens, heads, heads, 128), rows, threads=1)
+    want = zo.linear_batch(rb(mix.reshape(len(rows), heads * 128)), wr[3])
+    err = np.abs(got[rows].astype(np.float64) - want)
+    s = max(float(np.sqrt(np.mean(want.astype(np.float64) ** 2))), 1.0)
+    if err.max() > 2e-2 * s or err.mean() > 2e-3 * s:
+        raise RuntimeError(f"chain segment differs from the oracle chain on sampled rows: max {err.max():.3e} mean {err.mean():.3e}")
+    return {"rows": len(rows), "max_abs": float(err.max()), "mean_abs": float(err.mean()), "output_rms": s,
+            "oracle_s": time.perf_counter() - t0}
 
 
 def wide_main(args):
@@ -457,10 +494,20 @@ def other_paths(args):
     out = {}
     for name, steps in (("gemm", 200), ("chain", 60), ("wide", 60)):
         a = copy.copy(args)
-        a.path, a.steps, a.warmup, a.spinup_ms, a.no_cpu = name, steps, 10, 400.0, True
+        # the wide leg keeps its oracle check of 64 sampled rows (under a second of CPU work)
+        a.path, a.steps, a.warmup, a.spinup_ms, a.no_cpu = name, steps, 10, 400.0, name != "wide"
+        a.chain_heads, a.chain_check_rows = 0, 0
         line = PATH_MAINS[name](a)
         out[name] = {"workload": line["config"]["workload"], "value": line["value"], "ms_per_step": line["ms_per_step"],
                      "kernel_frac": line["roofline"]["frac"], "kernel": line["roofline"]["kernel"]}
+        if name == "wide":
+            out[name]["parity_check"] = line["cpu_baseline"]["sample"]
+        if name == "chain":
+            # the same segment at the full sequence length with 4 heads (hidden 512), where the
+            # oracle chain finishes in seconds: sampled output rows against it
+            a.chain_heads, a.chain_check_rows, a.steps, a.warmup, a.spinup_ms = 4, 8, 3, 1, 0.0
+            small = PATH_MAINS[name](a)
+            out[name]["parity_check"] = {"workload": small["config"]["workload"], **small["parity_check"]}
     return out
 
 
@@ -469,6 +516,9 @@ def main():
     ap.add_argument("--path", choices=["attention", "gemm", "chain", "wide"], default="attention",
                     help="attention (the headline metric) or the projection GEMM beside it")
     ap.add_argument("--wide-tokens", type=int, default=16384, help="--path wide: sequence length (multiple of 64)")
+    ap.add_argument("--chain-heads", type=int, default=0, help="--path chain: heads (hidden = 128 x heads); 0 = the model's 30")
+    ap.add_argument("--chain-check-rows", type=int, default=0,
+                    help="--path chain: check this many sampled output rows against the oracle chain (use with few heads)")
     ap.add_argument("--chain-act", choices=["bf16", "f32"], default="bf16",
                     help="--path chain: activation buffers as bf16, or f32 as the reference's chain keeps them")
     ap.add_argument("--m", type=int, default=4608)

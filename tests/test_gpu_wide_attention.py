@@ -64,6 +64,25 @@ def test_wide_head_reference_case_sampled_rows_and_rerun(ctx):
     assert (np.abs(got).max(axis=(1, 2)) > 0).all()
 
 
+def test_wide_head_at_the_1024_px_length_sampled_rows_and_rerun(ctx):
+    # 16384 tokens, the VAE mid-block of a 1024 px render and the length the kernel's throughput
+    # is quoted on: one workgroup per CU, no key ranges. Sampled rows in the manner of
+    # metal/mattn_test.zig:138-224 (both halves of the first, a middle and the last query tile,
+    # rows of every wave), N(0, 1) operands at the bf16 bar, byte-equal rerun.
+    tokens = 16384
+    rng = np.random.default_rng(0x16384)
+    q, k, v = draw(rng, tokens)
+    cfg = host.Config(tokens, 1, 1, 512)
+    got = ctx.run(q, k, v, cfg).reshape(tokens, 1, 512)
+    again = ctx.run(q, k, v, cfg).reshape(tokens, 1, 512)
+    assert got.tobytes() == again.tobytes()
+    assert np.isfinite(got).all()
+    rows = [0, 31, 32, 63, 64, 95, 96, 127, 128, 8191, 8192, 8255, 12345, 16256, 16319, 16352, 16383]
+    want = zo.attention_token_list(q, k, v, zo.Config(tokens, 1, 1, 512), rows)
+    refimpl.check_close(got[rows], want.reshape(len(rows), 1, 512), "wide head, 16384 tokens")
+    assert (np.abs(got).max(axis=(1, 2)) > 0).all()
+
+
 def test_wide_head_sharp_softmax_and_large_scores(ctx):
     # rows whose scores span a wide range (no QK-norm in front of this attention): a key along
     # the query's direction scores about 34 against a field of N(0, 1) scores; the running
