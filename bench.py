@@ -460,7 +460,7 @@ def wide_main(args):
         "config": {"workload": f"vae mid-block attention: tokens {tokens}, heads 1, head_dim 512, f32 in and out",
                    "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS, "untimed_spinup_launches": spun},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "attn_wide_kernel",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "attn_wide_kernel + wide_merge_kernel + attn_wide_safe_kernel (no tile flagged)",
                      "kernel_ms": kern_ms},
     }
     if not args.no_cpu:

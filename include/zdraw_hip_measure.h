@@ -36,6 +36,11 @@ void zdraw_hip_set_attention_variant(int variant);
  * each (default); 0 = eight waves, 64 x 128 each. */
 void zdraw_hip_set_gemm_build(int build);
 
+/* How many query tiles (128 rows) of the last wide-head launch had a score outgrow its row's
+ * fixed reference point and were formed again by the running-maximum kernel (waits for that
+ * launch). 0 on ordinary data; -1 if no wide-head launch has been made or the read failed. */
+int zdraw_hip_wide_redo_tiles(void);
+
 /* A queue as zdraw_hip_create_queue makes it, its stream confined to cu_count compute units
  * (0 < cu_count < the device's CU count; anything else: an ordinary queue): does a kernel's
  * time follow the CU count or the board's power limit. */

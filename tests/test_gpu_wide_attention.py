@@ -122,6 +122,40 @@ def test_wide_head_reference_point_moves_several_times(ctx):
         assert np.abs(want[i, 0] - v[1100 + n, 0]).max() < 1e-2  # the last planted key takes the row
 
 
+def test_wide_head_scores_that_outgrow_the_fixed_reference_take_the_safe_kernel(ctx):
+    # The fast kernel exponentiates every score of a row against the largest score of the first
+    # block of its key range and flags a query tile whose row sums show a score more than 2^90
+    # above that; flagged tiles are formed again by the running-maximum kernel that follows every
+    # launch. Ordinary data flags nothing; a key 75 nats (108 in log2) above a field of N(0, 1)
+    # scores, late in a range, flags its tile and only that one, and the rows still match.
+    L = hip.lib()
+    tokens = 1024
+    rng = np.random.default_rng(79)
+    q, k, v = draw(rng, tokens)
+    cfg = host.Config(tokens, 1, 1, 512)
+    got = ctx.run(q, k, v, cfg).reshape(tokens, 1, 512)
+    assert L.zdraw_hip_wide_redo_tiles() == 0
+    refimpl.check_close(got, zo.attention_run(q, k, v, zo.Config(tokens, 1, 1, 512)), "ordinary data")
+    # rows 300 and 301 (tile 2) lean on keys 900 and 901, row 900 (tile 7) on key 1000: keys in the fifth and
+    # the last block of the fourth key range (1024 tokens run as four ranges of eight blocks)
+    for i, j in ((300, 900), (301, 901), (900, 1000)):
+        k[j, 0] = 3.3 * q[i, 0] / np.linalg.norm(q[i, 0]) * np.sqrt(512.0)
+    got = ctx.run(q, k, v, cfg).reshape(tokens, 1, 512)
+    flagged = L.zdraw_hip_wide_redo_tiles()
+    assert flagged == 2, flagged
+    assert np.isfinite(got).all()
+    want = zo.attention_run(q, k, v, zo.Config(tokens, 1, 1, 512))
+    # (a bf16 operand's rounding error grows with the score: the planted rows are sharp one-hot
+    # rows and are compared as such; every other row at the usual bar)
+    others = np.ones(tokens, bool)
+    others[[300, 301, 900]] = False
+    refimpl.check_close(got[others], want[others], "rows beside the planted ones")
+    for i, j in ((300, 900), (301, 901), (900, 1000)):
+        assert np.abs(got[i, 0] - v[j, 0]).max() < 2e-2
+    again = ctx.run(q, k, v, cfg).reshape(tokens, 1, 512)
+    assert got.tobytes() == again.tobytes()
+
+
 def test_wide_head_refusals_leave_nothing_enqueued(ctx):
     L = hip.lib()
     d0 = L.zdraw_hip_dispatch_count()

@@ -27,3 +27,12 @@ def test_only_the_source_writes_m0_in_the_four_wave_gemm():
     # compiler does not know M0 is live between them, so it must not have put a write of its own there
     bad = build.m0_writes()
     assert not bad, "\n".join(bad[:20])
+
+
+@pytest.mark.skipif(not (os.path.exists("/opt/rocm/bin/hipcc") or shutil.which("hipcc")), reason="needs hipcc")
+def test_wide_head_kernel_keeps_its_accumulators_in_place_and_its_loop_free_of_spills():
+    # attn_wide.hip: every MFMA of attn_wide_kernel is an assembly statement with the accumulator
+    # tied to the result; nothing else may touch the accumulation file before the wait that ends a
+    # step, and the blocks that hold the MFMAs may not use scratch memory
+    bad = build.wide_mfma_hazards()
+    assert not bad, "\n".join(bad[:20])

@@ -95,10 +95,11 @@ def m0_writes(src: str = os.path.join(CSRC, "gemm_half.hip"), kernel_substr: str
     return bad
 
 
-def tied_mfma_hazards(src: str = os.path.join(CSRC, "gemm_half.hip"), extra_flags=()) -> list[str]:
-    """Compiles `src` to gfx950 assembly and lists every place where something other than
-    an MFMA touches an accumulation register while a hand-written v_mfma_f32_16x16x32 may
-    still be writing it. Those MFMAs are assembly statements, so the compiler adds none of
+def tied_mfma_hazards(src: str = os.path.join(CSRC, "gemm_half.hip"), extra_flags=(),
+                      mfma_prefix: str = "v_mfma_f32_16x16x32", kernel_substr: str = "") -> list[str]:
+    """Compiles `src` to gfx950 assembly and lists every place (in the kernels whose symbol
+    contains `kernel_substr`) where something other than an MFMA touches an accumulation
+    register while a hand-written MFMA (`mfma_prefix`) may still be writing it. Those MFMAs are assembly statements, so the compiler adds none of
     the wait states it adds after the builtin; the source instead ends every run of them
     with `s_nop 15` before control leaves the block. A copy or spill of an accumulator that
     the register allocator places inside such a run would read a stale value: this check
@@ -115,13 +116,51 @@ def tied_mfma_hazards(src: str = os.path.join(CSRC, "gemm_half.hip"), extra_flag
         if text.endswith(":") and not text.startswith("."):
             kernel, hot = text[:-1], False
             continue
+        if kernel_substr not in kernel:
+            continue
         op = text.split()[0]
-        if op.startswith("v_mfma_f32_16x16x32"):
+        if op.startswith(mfma_prefix):
             hot = True
         elif op == "s_nop" and text.split()[1] == "15":
             hot = False
         elif hot and agpr.search(text):
             bad.append(f"{kernel}: line {no}: {text}")
+    return bad
+
+
+def wide_mfma_hazards(extra_flags=()) -> list[str]:
+    """The same check for the wide-head kernel (attn_wide.hip, attn_wide_kernel): all of its MFMAs
+    are assembly statements, its 256 accumulation registers hold O^T for the whole walk, and every
+    step ends with the wait (`s_nop 15` ...) before anything else may read them. Also lists any
+    use of scratch memory inside a block that holds such MFMAs: the loop is written to fit the
+    register file exactly, and a spill there waits on every load in flight."""
+    import re
+    src = os.path.join(CSRC, "attn_wide.hip")
+    bad = tied_mfma_hazards(src, extra_flags, mfma_prefix="v_mfma_f32_32x32x16", kernel_substr="attn_wide_kernel")
+    lines = _device_asm(src, extra_flags)
+    kernel, block, mfmas, scratch = "", "", 0, []
+    label = re.compile(r"^([.\w$]+):")
+
+    def close():
+        if "attn_wide_kernel" in kernel and mfmas >= 32 and scratch:
+            bad.append(f"{kernel}: {len(scratch)} scratch accesses in {block} beside {mfmas} MFMAs, e.g. {scratch[0]}")
+
+    for line in lines:
+        text = line.split(";")[0].strip()
+        if not text:
+            continue
+        m = label.match(text)
+        if m:
+            close()
+            if not text.startswith("."):
+                kernel = m.group(1)
+            block, mfmas, scratch = m.group(1), 0, []
+            continue
+        if text.startswith("v_mfma"):
+            mfmas += 1
+        elif text.startswith("scratch_"):
+            scratch.append(text)
+    close()
     return bad
 
 
@@ -139,9 +178,9 @@ def build_host(verbose: bool = False) -> str:
 def check_hand_scheduled_kernels(verbose: bool = False):
     """The GEMM's hand-placed MFMAs and its M0 held across loads are safe only as long as the
     compiler puts nothing of its own in between: a toolchain that does fails the build here."""
-    bad = m0_writes() + tied_mfma_hazards()
+    bad = m0_writes() + tied_mfma_hazards() + wide_mfma_hazards()
     if bad:
-        raise RuntimeError("gemm_half.hip compiled to code that breaks its hand-written schedule:\n  " + "\n  ".join(bad))
+        raise RuntimeError("a kernel compiled to code that breaks its hand-written schedule:\n  " + "\n  ".join(bad))
     if verbose:
         print("hand-scheduled kernels: no foreign M0 write, no accumulator touched inside an MFMA run")
 

@@ -129,6 +129,8 @@ struct WideArgs {
     int32_t splits; // key ranges per query tile (wide_splits; 0 or 1: none); > 1 needs the two buffers below
     float* part_o;  // f32 [splits][tokens][512]: unnormalised O of each key range
     float* part_ml; // f32 [splits][tokens][2]: its reference point and row sum
+    int* redo;      // [wide_tiles(tokens)]: set by the kernel for a query tile (128 rows) whose scores outgrew the
+                    // fixed reference point; such tiles are formed again by the running-maximum kernel that follows
 };
 // f32 -> bf16 rounding of the three operands (Q with its scale) in one launch.
 struct WidePrepArgs {
@@ -136,13 +138,15 @@ struct WidePrepArgs {
     void* qo; void* ko; void* vo;
     int64_t chunks; // 8-element chunks per operand
     float q_scale;
-    int32_t pad0;
+    int32_t redo_tiles; // entries of redo that the launch clears
+    int* redo;
 };
 int wide_head_dim();
 int wide_block_rows();
 // Key ranges per query tile that fill a device of `cus` compute units (1: no split), and the
 // bytes of part_o followed by part_ml they need.
 int wide_splits(int tokens, int cus);
+int wide_tiles(int tokens); // query tiles (128 rows) = entries of WideArgs::redo
 size_t wide_part_bytes(int tokens, int splits);
 hipError_t launch_wide_round(const WidePrepArgs& args, hipStream_t stream);
 hipError_t launch_wide_attention(const WideArgs& args, hipStream_t stream);

@@ -766,6 +766,10 @@ int check_pipeline(void* pipeline, uint32_t kernel, int want_kind) {
 }
 
 bool g_wide_setup_done = false;
+// the redo flags of the last wide-head launch (measurement aid: how many tiles took the safe kernel)
+int* g_last_wide_redo = nullptr;
+int g_last_wide_tiles = 0;
+hipStream_t g_last_wide_stream = nullptr;
 
 // One wide head (metal/mattn.zig:261-275 widePick, :280-283 sdpaShape): f32 token-major
 // q, k, v, out [tokens][512] at byte offsets; rounds the operands into scratch slots 0-2,
@@ -805,8 +809,18 @@ int enqueue_wide(Queue* queue, void* q, void* k, void* v, void* out, const Zdraw
         }
         g_wide_setup_done = true;
     }
+    // one flag per query tile (scratch slot 4): set by the kernel where a row's scores outgrow its
+    // fixed reference point, cleared by the rounding launch, read by the kernel that forms such
+    // tiles again
+    Buffer* redo = queue_scratch(queue, 4, (size_t)wide_tiles((int)p->tokens) * sizeof(int));
+    if (!redo) {
+        set_err("scratch allocation failed");
+        return ZDRAW_HIP_ERR_HANDLE;
+    }
     WidePrepArgs pr;
     memset(&pr, 0, sizeof(pr));
+    pr.redo = static_cast<int*>(redo->ptr);
+    pr.redo_tiles = wide_tiles((int)p->tokens);
     pr.q = reinterpret_cast<const float*>(static_cast<const char*>(bs[0]->ptr) + in_off);
     pr.k = reinterpret_cast<const float*>(static_cast<const char*>(bs[1]->ptr) + in_off);
     pr.v = reinterpret_cast<const float*>(static_cast<const char*>(bs[2]->ptr) + in_off);
@@ -824,6 +838,7 @@ int enqueue_wide(Queue* queue, void* q, void* k, void* v, void* out, const Zdraw
     a.q = sc[0]->ptr; a.k = sc[1]->ptr; a.v = sc[2]->ptr;
     a.o = reinterpret_cast<float*>(static_cast<char*>(bs[3]->ptr) + out_off);
     a.tokens = (int32_t)p->tokens;
+    a.redo = static_cast<int*>(redo->ptr);
     a.splits = wide_splits(a.tokens, queue->dev->cus);
     if (a.splits > 1) {
         // a short sequence runs as key ranges whose shares go through scratch slot 3
@@ -848,6 +863,9 @@ int enqueue_wide(Queue* queue, void* q, void* k, void* v, void* out, const Zdraw
         g_trace_open.push_back(tp);
     }
     g_dispatch++;
+    g_last_wide_redo = a.redo;
+    g_last_wide_tiles = wide_tiles(a.tokens);
+    g_last_wide_stream = stream;
     return ZDRAW_HIP_OK;
 }
 
@@ -1787,6 +1805,16 @@ size_t zdraw_hip_clock_probe_read(uint64_t* cycles, uint64_t* ref_ticks, size_t 
 void zdraw_hip_set_attention_variant(int variant) { g_variant = variant & 3; }
 
 void zdraw_hip_set_gemm_build(int build) { gemm_set_build(build); }
+
+int zdraw_hip_wide_redo_tiles(void) {
+    if (!g_last_wide_redo || g_last_wide_tiles <= 0) return -1;
+    if (hipStreamSynchronize(g_last_wide_stream) != hipSuccess) return -1;
+    std::vector<int> flags((size_t)g_last_wide_tiles);
+    if (hipMemcpy(flags.data(), g_last_wide_redo, flags.size() * sizeof(int), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+    int n = 0;
+    for (int f : flags) n += f != 0;
+    return n;
+}
 
 void zdraw_hip_gemm_tail_plan(uint32_t m, uint32_t k, uint32_t n, uint32_t groups, uint32_t cus, uint32_t* tail_tiles,
                               uint32_t* splits) {

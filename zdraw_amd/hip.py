@@ -146,6 +146,7 @@ SYMBOLS = {
     "zdraw_hip_set_attention_variant": (None, [_int]),
     "zdraw_hip_set_gemm_build": (None, [_int]),
     "zdraw_hip_create_queue_on_cus": (_vp, [_vp, _int]),
+    "zdraw_hip_wide_redo_tiles": (_int, []),
     "zdraw_hip_attention_tail_plan": (None, [_u64, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "zdraw_hip_gemm_tail_plan": (None, [_u32, _u32, _u32, _u32, _u32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "zdraw_hip_zimage_axis_lens": (_int, [_u64, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
