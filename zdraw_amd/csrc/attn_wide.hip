@@ -610,33 +610,31 @@ __global__ void __launch_bounds__(NT, 1) attn_wide_safe_kernel(const WideArgs a)
 
 // Combines the key ranges of a split launch, in range order: with reference points m_p and row
 // sums l_p, O = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p, m = max_p m_p. A thread owns four
-// dims of one row; every range's load is sent before the first is used.
+// dims of one row; NP = the number of ranges is the build's, so that every range's load is sent
+// before the first is used, with no branch between them.
+template <int NP>
 __global__ void __launch_bounds__(256) wide_merge_kernel(const WideArgs a) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; // (row, dim / 4)
     const int64_t row = i / (WD / 4);
     if (row >= a.tokens) return;
     const int c4 = (int)(i - row * (WD / 4));
-    float m[kMaxSplits], l[kMaxSplits];
-    f32x4 o[kMaxSplits];
+    f32x2 ml[NP];
+    f32x4 o[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) ml[p] = *reinterpret_cast<const f32x2*>(a.part_ml + ((int64_t)p * a.tokens + row) * 2);
+#pragma unroll
+    for (int p = 0; p < NP; p++) o[p] = *reinterpret_cast<const f32x4*>(a.part_o + ((int64_t)p * a.tokens + row) * WD + 4 * c4);
     float mm = -INFINITY;
 #pragma unroll
-    for (int p = 0; p < kMaxSplits; p++)
-        if (p < a.splits) {
-            const f32x2 ml = *reinterpret_cast<const f32x2*>(a.part_ml + ((int64_t)p * a.tokens + row) * 2);
-            m[p] = ml[0];
-            l[p] = ml[1];
-            o[p] = *reinterpret_cast<const f32x4*>(a.part_o + ((int64_t)p * a.tokens + row) * WD + 4 * c4);
-            mm = fmaxf(mm, m[p]);
-        }
+    for (int p = 0; p < NP; p++) mm = fmaxf(mm, ml[p][0]);
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float lt = 0.f;
 #pragma unroll
-    for (int p = 0; p < kMaxSplits; p++)
-        if (p < a.splits) {
-            const float w = (m[p] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[p] - mm);
-            acc += o[p] * w;
-            lt += l[p] * w;
-        }
+    for (int p = 0; p < NP; p++) {
+        const float w = (ml[p][0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ml[p][0] - mm);
+        acc += o[p] * w;
+        lt += ml[p][1] * w;
+    }
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     *reinterpret_cast<f32x4*>(a.o + row * WD + 4 * c4) = acc * inv;
 }
@@ -680,7 +678,10 @@ hipError_t launch_wide_attention(const WideArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     if (nsp > 1) {
         const int64_t threads = (int64_t)a.tokens * (wide::WD / 4);
-        wide::wide_merge_kernel<<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream>>>(a);
+        const dim3 mgrid((unsigned)((threads + 255) / 256));
+        if (nsp == 2) wide::wide_merge_kernel<2><<<mgrid, dim3(256), 0, stream>>>(a);
+        else if (nsp == 4) wide::wide_merge_kernel<4><<<mgrid, dim3(256), 0, stream>>>(a);
+        else wide::wide_merge_kernel<8><<<mgrid, dim3(256), 0, stream>>>(a);
         if ((e = hipGetLastError()) != hipSuccess) return e;
     }
     // flagged tiles (none on ordinary data) are formed again, over whatever the launches above left there
