@@ -66,6 +66,40 @@ def test_noalloc_entry_matches_the_allocating_entry_on_shrinking_calls(ctx):
         assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), name
 
 
+def test_noalloc_entry_takes_no_device_memory_on_a_new_queue_with_weights_it_sees_first(ctx):
+    import torch
+
+    L = hip.lib()
+    # kernels loaded and the device's array looked up: one pass on the shared queue
+    warm = wl.Resident(ctx, _klein(6, 2, (20, 30), 100), dtype=hip.BF16, k_site=hip.K_PREPASS, bounded=True)
+    _both(ctx, warm)
+    warm.release()
+    # a second context: its queue has run nothing, its weight buffers are new to the library
+    # (their maxima, which the bounded softmax needs, are read during the call below)
+    c2 = host.Context.init()
+    try:
+        res = wl.Resident(c2, _klein(7, 2, (24, 26), 76), dtype=hip.BF16, k_site=hip.K_PREPASS, bounded=True)
+        res.o.write(np.full(res.o.nbytes, 0x7B, np.uint8))
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        b = L.zdraw_hip_batch_begin(c2.queue)
+        assert b
+        say("no-alloc: new queue, new weights")
+        rc = L.zdraw_hip_run_attention_fused_noalloc_enc(b, res.q.handle, res.k.handle, res.v.handle, res.o.handle,
+                                                         C.byref(res.params), C.byref(res.ext), C.byref(res.ops))
+        assert L.zdraw_hip_batch_end(b) == 0
+        assert rc == 0, hip.last_error()
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0, "the call changed the device's free memory"
+        got = res.read_output()
+        want = _both(c2, res)[0]  # the allocating entry, afterwards
+        res.release()
+        assert np.isfinite(want).all() and (np.abs(want).max(axis=-1) > 0).all()
+        assert np.array_equal(want.view(np.uint32), got.view(np.uint32))
+    finally:
+        c2.deinit()
+
+
 def test_noalloc_entry_refuses_what_does_not_fit_its_array(ctx):
     L = hip.lib()
     # bf16 Q' and K' of B x H x S rows: 512 bytes per row; 138240 rows do not fit 64 MiB
