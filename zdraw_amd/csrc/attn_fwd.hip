@@ -165,18 +165,23 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     // XCD-aware remap: consecutive logical ids (one head's query blocks) share an XCD's L2
     int logical;
     int split = 0;
-    if (a.splits > 1) {
+    int splits = 1; // parts of this workgroup's tile
+    if ((int)blockIdx.x < a.part_wgs) {
         // key-split tail: consecutive ids are the parts of one tile
         const int t = (int)blockIdx.x / a.splits;
+        if (t >= a.nqb * a.heads * a.batch - a.tile_base) return; // padding up to a multiple of 8
         split = (int)blockIdx.x - t * a.splits;
+        splits = a.splits;
         logical = a.tile_base + t;
     } else {
-        const int nwg = gridDim.x;
-        const int xcd = blockIdx.x & 7;
-        const int idx = blockIdx.x >> 3;
+        // (part_wgs is a multiple of 8, so a workgroup's XCD is its id's low bits here too)
+        const int w = (int)blockIdx.x - a.part_wgs;
+        const int nwg = (int)gridDim.x - a.part_wgs;
+        const int xcd = w & 7;
+        const int idx = w >> 3;
         const int base = nwg >> 3;
         const int rem = nwg & 7;
-        logical = a.tile_base + idx + xcd * base + (xcd < rem ? xcd : rem);
+        logical = idx + xcd * base + (xcd < rem ? xcd : rem);
     }
     const int bh = logical / a.nqb;
     const int qb = logical - bh * a.nqb;
@@ -227,8 +232,8 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
     }
     // a key-split workgroup walks positions [i0, i0 + nblk) of the list
     int i0 = 0;
-    if (a.splits > 1) {
-        const int per = (nblk + a.splits - 1) / a.splits;
+    if (splits > 1) {
+        const int per = (nblk + splits - 1) / splits;
         i0 = split * per;
         nblk = max(min(nblk - i0, per), 0);
     }
@@ -979,7 +984,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
 #pragma unroll
         for (int r = 0; r < 2; r++)
             inv_r[r] = __uint_as_float((unsigned)__builtin_amdgcn_ds_bpermute(4 * (16 * r + c16), (int)__float_as_uint(inv_l)));
-        if (a.splits > 1) {
+        if (splits > 1) {
             // unnormalised rows, reference point and denominator of this part
             const int64_t prow0 = (int64_t)blockIdx.x * BQ + wave * QR;
 #pragma unroll
@@ -1039,7 +1044,7 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             const float l_tot = pair_sum(l_run[qi]);
             const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
             const int qrow = q0 + 32 * qi + l32;
-            if (a.splits > 1) {
+            if (splits > 1) {
                 // unnormalised rows, reference point and denominator of this part
                 const int64_t prow = ((int64_t)blockIdx.x * BQ + wave * QR + 32 * qi + l32);
                 float* op = a.part_o + prow * D;
@@ -1103,9 +1108,11 @@ __global__ void __launch_bounds__(NW * 64, (QB == 2 ? 1 : 2)) attn_fwd_kernel(co
             }
         }
     }
-    if (a.clock_probe && tid == 0 && (int64_t)blockIdx.x < a.clock_cap) {
-        a.clock_probe[2 * blockIdx.x] = __builtin_readcyclecounter() - clk_c0;
-        a.clock_probe[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - clk_r0;
+    // (whole tiles only: the parts carry no probe)
+    const int64_t probe_slot = (int64_t)blockIdx.x - a.part_wgs;
+    if (a.clock_probe && tid == 0 && probe_slot >= 0 && probe_slot < a.clock_cap) {
+        a.clock_probe[2 * probe_slot] = __builtin_readcyclecounter() - clk_c0;
+        a.clock_probe[2 * probe_slot + 1] = __builtin_amdgcn_s_memrealtime() - clk_r0;
     }
 }
 
@@ -1167,7 +1174,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const AttnArgs a, int b
     }
 }
 
-// Whole tiles first, then (tail.splits > 1) the tiles of the last round in parts, then the merge.
+// One launch: the tiles of the last round in parts (tail.splits > 1), the whole tiles behind them; then the merge.
 template <typename TIn, int KMODE, bool MASKED, bool BOUNDED, int QB, int NW>
 static void launch_kernel(const AttnArgs& a, unsigned grid, hipStream_t stream) {
     if constexpr (std::is_same<TIn, bf16_t>::value && KMODE == kQkNone && QB == 1 && NW == 8) {
@@ -1187,21 +1194,17 @@ static hipError_t launch_one(const AttnArgs& a0, hipStream_t stream) {
     if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
     const int tail = a0.splits > 1 ? a0.tile_base : 0; // the planner leaves the tail size in tile_base
     AttnArgs a = a0;
-    a.tile_base = 0;
-    a.splits = 1;
     const int64_t whole = nwg - tail;
-    if (whole > 0) {
-        launch_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>(a, (unsigned)whole, stream);
+    a.tile_base = (int32_t)whole;
+    a.splits = tail > 0 ? a0.splits : 1;
+    a.part_wgs = tail > 0 ? (int32_t)(((int64_t)tail * a0.splits + 7) & ~(int64_t)7) : 0;
+    if (whole + a.part_wgs > 0x7fffffff) return hipErrorInvalidValue;
+    launch_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>(a, (unsigned)(whole + a.part_wgs), stream);
+    {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     if (tail > 0) {
-        a.tile_base = (int32_t)whole;
-        a.splits = a0.splits;
-        a.clock_probe = nullptr;
-        launch_kernel<TIn, KMODE, MASKED, BOUNDED, QB, NW>(a, (unsigned)(tail * a0.splits), stream);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
         const int rows = tail * NW * 32 * QB;
         const dim3 mgrid((unsigned)((rows + 7) / 8));
         if (a.splits <= 4) attn_merge_kernel<4><<<mgrid, dim3(256), 0, stream>>>(a, NW * 32 * QB);

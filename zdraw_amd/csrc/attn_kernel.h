@@ -70,11 +70,18 @@ struct AttnArgs {
     // cycles at [2i] and as ticks of the fixed 100 MHz reference at [2i+1], i < clock_cap
     unsigned long long* clock_probe;
     int64_t clock_cap;
-    // Key-split launches (splits > 1): workgroup id = (tile - tile_base) * splits + z; split z
-    // walks the z-th part of the tile's key-block list and writes its unnormalised O^T rows,
-    // reference point and denominator; attn_merge_kernel combines them in z order.
-    int32_t tile_base;  // first logical tile (segment, head, query block) of this launch
+    // One launch holds the tiles of the last, thinly filled round in parts (splits > 1) and the
+    // whole tiles behind them: workgroups below part_wgs are parts, id = (tile - tile_base) *
+    // splits + z (ids from (tiles - tile_base) * splits up to part_wgs are padding and return at
+    // once); part z walks the z-th share of the tile's key-block list and writes its
+    // unnormalised O^T rows, reference point and denominator, and attn_merge_kernel combines
+    // them in z order. Workgroups from part_wgs on take the whole tiles 0 .. tile_base - 1. The
+    // parts come first: they are short and mostly wait on memory, which the whole tiles that
+    // follow them onto the CUs cover.
+    int32_t tile_base;  // first logical tile (segment, head, query block) that is split
     int32_t splits;     // 0 or 1 = none
+    int32_t part_wgs;   // workgroups at the head of the grid that are parts (a multiple of 8), or 0
+    int32_t pad2;
     float* part_o;      // f32 [tile - tile_base][splits][block rows][128]
     float* part_ml;     // f32 [tile - tile_base][splits][block rows][2]
 };
