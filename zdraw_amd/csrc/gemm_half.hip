@@ -243,10 +243,9 @@ __device__ __forceinline__ void store_tile_lds16(const GemmArgs& g, void* c, con
 
 // XCD-aware tile id: workgroups go to the XCDs in turn, so each XCD gets one contiguous
 // run of the tile sequence
-__device__ __forceinline__ int logical_tile() {
-    const int nwg = gridDim.x;
-    const int xcd = blockIdx.x & 7;
-    const int idx = blockIdx.x >> 3;
+__device__ __forceinline__ int logical_tile(int wg, int nwg) {
+    const int xcd = wg & 7;
+    const int idx = wg >> 3;
     const int base = nwg >> 3;
     const int rem = nwg & 7;
     return idx + xcd * base + (xcd < rem ? xcd : rem);
@@ -286,7 +285,7 @@ __global__ void __launch_bounds__(NT, 2) gemm_kernel(const GemmArgs g) {
     const int h = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
 
-    const int logical = logical_tile();
+    const int logical = logical_tile((int)blockIdx.x, (int)gridDim.x);
     const int tiles_row = g.tiles_n * g.groups;
     int tm, tn;
     tile_coords(logical, (g.m + BM - 1) / BM, tiles_row, tm, tn);
@@ -418,7 +417,7 @@ __global__ void __launch_bounds__(WM * WN * 64, 2) gemm_dma_kernel(const GemmArg
     const int c16 = lane & 15;
     const int q4 = lane >> 4;
     const int wm = wave / WN, wn = wave % WN;
-    const int logical = logical_tile();
+    const int logical = logical_tile((int)blockIdx.x, (int)gridDim.x);
     const int tiles_row = g.tiles_n * g.groups;
     int tm, tn;
     tile_coords(logical, (g.m + TB - 1) / TB, tiles_row, tm, tn);
@@ -540,17 +539,21 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
     const int q4 = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
     // a tile of the split last round: workgroup = (tile, part), the part is a range of slabs
-    int logical, part_id = 0;
-    if (g.splits > 1) {
+    int logical, part_id = 0, splits = 1;
+    const int tiles_row = g.tiles_n * g.groups;
+    const int tiles_m = (g.m + BM - 1) / BM;
+    if ((int)blockIdx.x < g.part_wgs) {
         const int t = (int)blockIdx.x / g.splits;
+        if (t >= tiles_m * tiles_row - g.tile_base) return; // padding up to a multiple of 8
         part_id = (int)blockIdx.x - t * g.splits;
+        splits = g.splits;
         logical = g.tile_base + t;
     } else {
-        logical = logical_tile();
+        // (part_wgs is a multiple of 8, so a workgroup's XCD is its id's low bits here too)
+        logical = logical_tile((int)blockIdx.x - g.part_wgs, (int)gridDim.x - g.part_wgs);
     }
-    const int tiles_row = g.tiles_n * g.groups;
     int tm, tn;
-    tile_coords(logical, (g.m + BM - 1) / BM, tiles_row, tm, tn);
+    tile_coords(logical, tiles_m, tiles_row, tm, tn);
     const int grp = tn / g.tiles_n;
     tn -= grp * g.tiles_n;
     const void* const wp = grp == 0 ? g.w : g.w_more[grp - 1];
@@ -579,8 +582,8 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         w_off[j] = ((unsigned)wr * (unsigned)g.ldw + (unsigned)(c * 8)) * 2u + kBias - (unsigned)(j & 3) * 1024u;
     }
     int nslab = g.k / BK, slab0 = 0;
-    if (g.splits > 1) {
-        const int per = (nslab + g.splits - 1) / g.splits;
+    if (splits > 1) {
+        const int per = (nslab + splits - 1) / splits;
         slab0 = part_id * per;
         nslab = max(min(nslab - slab0, per), 0);
     }
@@ -681,7 +684,7 @@ __global__ void __launch_bounds__(256, 1) gemm_ring_kernel(const GemmArgs g) {
         mfma16_drain();
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // no direct load may outlive the workgroup's LDS
-    if (g.splits > 1) {
+    if (splits > 1) {
         // partial tile in the accumulation layout: [tile][part][wave][i][j][lane] x 16 bytes,
         // every store instruction 1 KB in a row; the merge kernel reads it the same way
         f32x4* dst = reinterpret_cast<f32x4*>(g.part) +
@@ -832,21 +835,16 @@ static hipError_t launch_one(const GemmArgs& g0, hipStream_t stream) {
     if (nwg <= 0 || nwg > 0x7fffffff) return hipErrorInvalidValue;
     if constexpr (!std::is_same<TA, float>::value) {
         if (g_gemm_build == 1 && g.k % BK == 0) {
-            // whole tiles first, then (splits > 1) the tiles of the last round in parts, then the merge
+            // one launch: (splits > 1) the tiles of the last round in parts, the whole tiles behind them; then the merge
             const int tail = g0.splits > 1 ? g0.tile_base : 0; // the planner leaves the tail size in tile_base
             if (tail < 0 || tail > nwg || g0.splits > kMaxKSplits || (tail > 0 && g0.part == nullptr)) return hipErrorInvalidValue;
-            g.tile_base = 0;
-            g.splits = 1;
             const int64_t whole = nwg - tail;
-            if (whole > 0) {
-                gemm_ring_kernel<F16, TC><<<dim3((unsigned)whole), dim3(256), kRingLdsBytes, stream>>>(g);
-                hipError_t e = hipGetLastError();
-                if (e != hipSuccess) return e;
-            }
+            g.tile_base = (int32_t)whole;
+            g.splits = tail > 0 ? g0.splits : 1;
+            g.part_wgs = tail > 0 ? (int32_t)(((int64_t)tail * g0.splits + 7) & ~(int64_t)7) : 0;
+            if (whole + g.part_wgs > 0x7fffffff) return hipErrorInvalidValue;
+            gemm_ring_kernel<F16, TC><<<dim3((unsigned)(whole + g.part_wgs)), dim3(256), kRingLdsBytes, stream>>>(g);
             if (tail > 0) {
-                g.tile_base = (int32_t)whole;
-                g.splits = g0.splits;
-                gemm_ring_kernel<F16, TC><<<dim3((unsigned)(tail * g0.splits)), dim3(256), kRingLdsBytes, stream>>>(g);
                 hipError_t e = hipGetLastError();
                 if (e != hipSuccess) return e;
                 gemm_merge_kernel<F16, TC><<<dim3((unsigned)tail * 16u), dim3(256), 0, stream>>>(g);

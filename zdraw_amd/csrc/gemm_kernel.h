@@ -20,12 +20,16 @@ struct GemmArgs {
     const void* w_more[2];
     void* c_more[2];
     // Tiles of a partly filled last round, split along k (set by the caller from gemm_tail_plan;
-    // splits <= 1: none). On entry tile_base holds the NUMBER of tail tiles; the launcher runs
-    // the whole tiles first, then the tail tiles in `splits` parts each (fp32 partial tiles to
-    // `part`), then the kernel that adds the parts in part order and writes C.
+    // splits <= 1: none). On entry tile_base holds the NUMBER of tail tiles; the launcher puts
+    // the tail tiles, in `splits` parts each (fp32 partial tiles to `part`), at the head of the
+    // one launch (part_wgs workgroups, a multiple of 8; ids past the last part return at once)
+    // with the whole tiles behind them, which cover the parts' waits as they follow them onto
+    // the CUs; then the kernel that adds the parts in part order and writes C.
     int32_t tile_base;
     int32_t splits;
     float* part;
+    int32_t part_wgs; // set by the launcher
+    int32_t pad1;
     // f32 activations: room for A rounded to the weight's type, [m][k] 16-bit (gemm_round_bytes
     // says how much; null: A is rounded block by block on its way into LDS instead)
     void* a16;
