@@ -320,8 +320,12 @@ def test_full_configs_sampled_rows_and_bit_stability(ctx, name, nsample):
     res.k_site = hip.K_PREPASS
     res.ext.k_site = hip.K_PREPASS
     pre = res.run()
+    bound = res.ext.score_bound
     res.ext.score_bound = 0.0  # running-maximum softmax
     dyn = res.run()
+    res.ext.score_bound = bound
+    res.ext.staging = hip.F16  # prepared Q and K staged as IEEE half, scores on the f16 MFMA
+    half = res.run()
     res.release()
     toks = refimpl.sample_tokens(w, nsample)
     say(f"  oracle on {len(toks)} query tokens x {w.batch} segments")
@@ -332,7 +336,9 @@ def test_full_configs_sampled_rows_and_bit_stability(ctx, name, nsample):
     say(f"  pre-pass  K: max abs {mx:.2e} mean abs {mean:.2e}")
     mx, mean = refimpl.check_close(dyn[:, toks], want, name + " (running maximum)")
     say(f"  running max: max abs {mx:.2e} mean abs {mean:.2e}")
-    assert np.isfinite(got).all() and np.isfinite(pre).all()
+    mx, mean = refimpl.check_close(half[:, toks], want, name + " (half staging)")
+    say(f"  half staging: max abs {mx:.2e} mean abs {mean:.2e}")
+    assert np.isfinite(got).all() and np.isfinite(pre).all() and np.isfinite(half).all()
     # no row left unwritten: every output row has a non-zero element
     assert (np.abs(got).max(axis=-1) > 0).all()
 
